@@ -1,0 +1,81 @@
+// Shared declarations of the gfx950 2-simplicial attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sa2.h"
+
+namespace sa2 {
+
+// One [B,N,H,D] tensor: base pointer and element strides (D stride is 1).
+struct Tensor {
+    void* p;
+    int64_t sb, sn, sh;
+    __host__ __device__ int64_t off(int b, int n, int h) const { return b * sb + n * sn + h * sh; }
+};
+
+// Everything a kernel needs about one call.  w1/w2 are already the inclusive
+// window reaches: query i sees keys [i-w, i].
+struct Problem {
+    int B, N, H, D;
+    int w1, w2;
+    float scale, k2_bias, v2_bias;
+    Tensor q, k1, k2, v1, v2, out, dout;
+    Tensor dq, dk1, dk2, dv1, dv2;   // p == nullptr: not requested
+    float* lse;                      // [B,H,N]
+    float* dsum;                     // [B,H,N]  sum_d dout*out
+    void* scratch;                   // remaining workspace (path specific)
+    size_t scratch_bytes;
+};
+
+// ---- element loads / stores -------------------------------------------------
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+__device__ __forceinline__ float to_float(f16_t x) { return (float)x.v; }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);   // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                             // round to nearest even
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ void from_float(float f, float* p) { *p = f; }
+__device__ __forceinline__ void from_float(float f, bf16_t* p) { p->bits = f32_to_bf16_bits(f); }
+__device__ __forceinline__ void from_float(float f, f16_t* p) { p->v = (_Float16)f; }
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// log(sum_w + 1e-8) from the running maximum m and l = sum exp(s-m), for any m.
+__device__ __forceinline__ float lse_with_eps(float m, float l) {
+    const float log_eps = -18.420680743952367f;   // log(1e-8)
+    if (m > log_eps) return m + logf(l + 1e-8f * expf(-m));
+    return log_eps + log1pf(l * expf(m - log_eps));
+}
+
+// ---- launchers (each returns a sa2_status) ----------------------------------
+int launch_rowdot(const Tensor& out, const Tensor& dout, float* dsum, int B, int N, int H, int D,
+                  int dtype, hipStream_t st);
+int launch_generic_fwd(const Problem& p, int dtype, hipStream_t st);
+int launch_generic_bwd(const Problem& p, int dtype, hipStream_t st);
+size_t generic_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
+
+bool mfma_supported(int B, int N, int H, int D, int w1, int w2, int dtype);
+bool mfma_layout_ok(const Problem& p, bool backward);
+int launch_mfma_fwd(const Problem& p, hipStream_t st);
+int launch_mfma_bwd(const Problem& p, hipStream_t st);
+size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
+
+}  // namespace sa2

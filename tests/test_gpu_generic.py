@@ -1,0 +1,197 @@
+"""GPU parity of the generic fp32-FMA kernels against the CPU oracle, through
+the C ABI.  Shapes, dtypes, windows, biases and edge cases re-express the
+reference's own correctness suite (simplicial/test_correctness.py:148-455) with
+N(0,1)-sized inputs where the reference used 0.1*N(0,1)."""
+import math
+
+import pytest
+import torch
+
+from oracle import simplicial_oracle as orc
+from tests.util import assert_close_rel, make_inputs, oracle_all, rel_err, run_device
+
+pytestmark = pytest.mark.gpu
+GENERIC = 1
+
+
+def test_config1_fp32_forward_matches_literal_oracle():
+    """BASELINE config 1: fp32, B1 H2 N128 D64, w 32/16, seed 0, rtol = atol = 1e-5
+    against the literal-order fp32 loop and against the fp64 truth."""
+    inp = make_inputs(1, 128, 2, 64, seed=0)
+    got = run_device(inp, 32, 16, flags=GENERIC, backward=False)
+    lit = orc.literal_loop(*inp[:5], 32, 16)
+    assert torch.allclose(got["out"].cpu(), lit, rtol=1e-5, atol=1e-5)
+    o64, lse64 = orc.forward_windowed(*[x.double() for x in inp[:5]], 32, 16)
+    assert torch.allclose(got["out"].cpu().double(), o64, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(got["lse"].cpu().double(), lse64, rtol=1e-5, atol=1e-5)
+
+
+def test_config1_fp32_gradients():
+    inp = make_inputs(1, 128, 2, 64, seed=0)
+    got = run_device(inp, 32, 16, flags=GENERIC)
+    want = oracle_all(inp, 32, 16)
+    for name in ("dq", "dk1", "dk2", "dv1", "dv2"):
+        assert torch.allclose(got[name].cpu().double(), want[name], rtol=1e-5, atol=1e-5), name
+
+
+@pytest.mark.parametrize("shape", [(1, 32, 1, 16), (2, 64, 2, 32), (4, 128, 4, 64), (1, 256, 8, 128), (1, 40, 2, 256),
+                                   (2, 37, 3, 20)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_forward_backward_vs_oracle(shape, dtype):
+    """simplicial/test_correctness.py:148-177 (w1 = w2 = 16), plus gradients."""
+    B, N, H, D = shape
+    inp = make_inputs(B, N, H, D, seed=N + D, dtype=dtype, mag=0.5)
+    got = run_device(inp, 16, 16, flags=GENERIC)
+    want = oracle_all(inp, 16, 16)
+    tol = 1e-5 if dtype == torch.float32 else (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    for name in ("out", "dq", "dk1", "dk2", "dv1", "dv2"):
+        assert_close_rel(got[name], want[name], tol, name)
+    assert_close_rel(got["lse"], want["lse"], 1e-5, "lse")
+
+
+@pytest.mark.parametrize("w", [(1, 1), (4, 4), (8, 3), (0, 5), (5, 0), (0, 0), (64, 64), (100, 7), (70, 200)])
+def test_window_sizes(w):
+    """simplicial/test_correctness.py:179-198 and the w = 1 / w > N edge cases (324-354)."""
+    inp = make_inputs(2, 96, 2, 32, seed=7)
+    got = run_device(inp, w[0], w[1], flags=GENERIC)
+    want = oracle_all(inp, w[0], w[1])
+    for name in ("out", "lse", "dq", "dk1", "dk2", "dv1", "dv2"):
+        assert_close_rel(got[name], want[name], 2e-5, name)
+
+
+@pytest.mark.parametrize("bias", [(0.0, 0.0), (0.1, 0.2), (-0.1, -0.2), (1.0, 0.5)])
+def test_bias_values(bias):
+    """simplicial/test_correctness.py:200-226."""
+    inp = make_inputs(2, 64, 2, 32, seed=11)
+    got = run_device(inp, 16, 8, None, bias[0], bias[1], flags=GENERIC)
+    want = oracle_all(inp, 16, 8, None, bias[0], bias[1])
+    for name in ("out", "lse", "dq", "dk1", "dk2", "dv1", "dv2"):
+        assert_close_rel(got[name], want[name], 2e-5, name)
+
+
+def test_zero_and_extreme_inputs():
+    """simplicial/test_correctness.py:356-396: all-zero inputs, and all-10.0
+    inputs (logits of 4000) stay finite and equal the analytic answer."""
+    dev = torch.device("cuda:0")
+    import simplical_attn_amd as sa
+    z = torch.zeros(1, 32, 2, 16, device=dev)
+    out, lse = sa.simplicial_forward(z, z, z, z, z, 8, 8, flags=GENERIC)
+    assert torch.equal(out, torch.zeros_like(out))
+    want = torch.tensor([math.log((min(i, 8) + 1) ** 2 + 1e-8) for i in range(32)])
+    assert torch.allclose(lse[0, 0].cpu(), want.float(), rtol=1e-6)
+    t = torch.full((1, 32, 2, 16), 10.0, device=dev)
+    out, lse = sa.simplicial_forward(t, t, t, t, t, 8, 8, flags=GENERIC)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert torch.allclose(out, torch.full_like(out, 100.0), rtol=1e-5)
+
+
+def test_epsilon_dominates_for_very_negative_logits():
+    """Row 0 with one very negative logit: O -> 0 and LSE -> log(1e-8) as the
+    oracle's +1e-8 demands (simplicial/reference.py:74)."""
+    inp = make_inputs(1, 8, 1, 16, seed=3, mag=3.0)
+    q, k1, k2 = inp[0], inp[1], inp[2]
+    sign = torch.sign((q[:, 0] * k1[:, 0] * k2[:, 0]).sum(-1, keepdim=True))
+    inp[0][:, 0] = -q[:, 0] * sign * 50.0
+    got = run_device(inp, 4, 4, 1.0, flags=GENERIC, backward=False)
+    o64, lse64 = orc.forward_windowed(*[x.double() for x in inp[:5]], 4, 4, 1.0)
+    assert torch.allclose(got["out"].cpu().double(), o64, rtol=1e-4, atol=1e-6)
+    assert torch.allclose(got["lse"].cpu().double(), lse64, rtol=1e-5, atol=1e-5)
+    assert abs(got["lse"][0, 0, 0].item() - math.log(1e-8)) < 1e-3
+
+
+def test_deterministic_and_gradient_accumulation():
+    """simplicial/test_correctness.py:290-318, 402-421: two runs give identical
+    bits; a second backward doubles .grad."""
+    inp = make_inputs(2, 80, 2, 32, seed=42)
+    a = run_device(inp, 12, 6, flags=GENERIC)
+    b = run_device(inp, 12, 6, flags=GENERIC)
+    for name in a:
+        assert torch.equal(a[name], b[name]), name
+    from simplical_attn_amd import TwoSimplicialAttention
+    dev = torch.device("cuda:0")
+    leaves = [x.to(dev).requires_grad_(True) for x in inp[:5]]
+    attn = TwoSimplicialAttention(32, 12, 6)
+    attn(*leaves).sum().backward()
+    first = [x.grad.clone() for x in leaves]
+    attn(*leaves).sum().backward()
+    for g, x in zip(first, leaves):
+        assert torch.allclose(x.grad, 2 * g, atol=1e-4)
+
+
+def test_finite_differences():
+    """simplicial/test_correctness.py:256-288 re-expressed: central differences
+    of sum(O*dO) on sampled elements, fp32 inputs."""
+    from simplical_attn_amd import TwoSimplicialAttention
+    dev = torch.device("cuda:0")
+    inp = make_inputs(1, 16, 1, 8, seed=5, mag=0.7)
+    dout = inp[5].to(dev)
+    attn = TwoSimplicialAttention(8, 4, 4)
+    got = run_device(inp, 4, 4, flags=GENERIC)
+    base = [x.to(dev) for x in inp[:5]]
+    g = torch.Generator().manual_seed(0)
+    eps = 1e-2
+    for t, name in enumerate(("dq", "dk1", "dk2", "dv1", "dv2")):
+        flat_idx = torch.randperm(base[t].numel(), generator=g)[:12]
+        for idx in flat_idx.tolist():
+            plus = [x.clone() for x in base]
+            minus = [x.clone() for x in base]
+            plus[t].view(-1)[idx] += eps
+            minus[t].view(-1)[idx] -= eps
+            num = ((attn(*plus) * dout).sum() - (attn(*minus) * dout).sum()).item() / (2 * eps)
+            ana = got[name].view(-1)[idx].item()
+            assert abs(num - ana) <= 2e-2 * max(1.0, abs(ana)), (name, idx, num, ana)
+
+
+def test_strided_inputs_and_needs_input_grad():
+    """Per-tensor strides (a packed [B,N,5,H,D] projection sliced five ways) and
+    gradients requested for a subset of the inputs (triton_impl.py:73-77)."""
+    from simplical_attn_amd import TwoSimplicialAttentionFunction as Fn
+    dev = torch.device("cuda:0")
+    B, N, H, D = 2, 48, 2, 32
+    inp = make_inputs(B, N, H, D, seed=9)
+    packed = torch.stack(inp[:5], dim=2).to(dev)            # [B,N,5,H,D]
+    views = [packed[:, :, t] for t in range(5)]
+    assert not views[0].is_contiguous()
+    leaves = [v.detach().requires_grad_(t in (0, 2, 3)) for t, v in enumerate(views)]
+    out = Fn.apply(*leaves, 8, 5, None, 0.0, 0.0)
+    out.backward(inp[5].to(dev))
+    want = oracle_all(inp, 8, 5)
+    assert_close_rel(out.detach(), want["out"], 2e-5, "out")
+    assert leaves[1].grad is None and leaves[4].grad is None
+    for t, name in ((0, "dq"), (2, "dk2"), (3, "dv1")):
+        assert_close_rel(leaves[t].grad, want[name], 2e-5, name)
+
+
+def test_half_open_window_convention():
+    """window_inclusive = 0 masks (i-w, i] like the reference's device kernels
+    (simplicial/kernels.py:133-136): equal to the closed window with w-1."""
+    import simplical_attn_amd as sa
+    dev = torch.device("cuda:0")
+    inp = [x.to(dev) for x in make_inputs(1, 40, 2, 16, seed=13, with_dout=False)]
+    a, la = sa.simplicial_forward(*inp, 6, 4, flags=GENERIC, window_inclusive=False)
+    b, lb = sa.simplicial_forward(*inp, 5, 3, flags=GENERIC, window_inclusive=True)
+    assert torch.equal(a, b) and torch.equal(la, lb)
+
+
+def test_error_codes():
+    from simplical_attn_amd import _lib, simplicial_forward
+    dev = torch.device("cuda:0")
+    x = torch.zeros(1, 8, 1, 260, device=dev)
+    with pytest.raises(_lib.Sa2Error) as e:
+        simplicial_forward(x, x, x, x, x, 4, 4)
+    assert e.value.status == -3
+    y = torch.zeros(1, 8, 1, 16, device=dev)
+    with pytest.raises(_lib.Sa2Error) as e:
+        simplicial_forward(y, y, y, y, y, -1, 4)
+    assert e.value.status == -5
+    with pytest.raises(RuntimeError):
+        simplicial_forward(y.cpu(), y.cpu(), y.cpu(), y.cpu(), y.cpu(), 4, 4)
+
+
+def test_rowdot():
+    from simplical_attn_amd import compute_D_kernel
+    dev = torch.device("cuda:0")
+    a = torch.randn(2, 33, 3, 40, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(2, 33, 3, 40, device=dev, dtype=torch.bfloat16)
+    want = (a.float() * b.float()).sum(-1).permute(0, 2, 1)
+    assert torch.allclose(compute_D_kernel(a, b), want, rtol=1e-5, atol=1e-5)
