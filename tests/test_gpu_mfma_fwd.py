@@ -1,0 +1,113 @@
+"""GPU parity of the bf16 MFMA forward kernel, through the C ABI.
+
+Tolerance (bf16 path): max|diff| <= 2e-2 * max|ref| per tensor against the
+fp64 oracle evaluated on the same bf16-rounded inputs.  Large shapes are
+checked against the oracle on row ranges (the oracle is O(T) on the CPU) and,
+over the whole tensor, against the generic fp32 kernels, which the small-shape
+tests tie to the oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import simplicial_oracle as orc
+from tests.util import assert_close_rel, make_inputs
+
+pytestmark = pytest.mark.gpu
+GENERIC, MFMA = 1, 2
+BF16_TOL = 2e-2
+
+
+def fwd(inp, w1, w2, scale=None, kb=0.0, vb=0.0, flags=MFMA):
+    import simplical_attn_amd as sa
+    dev = torch.device("cuda:0")
+    return sa.simplicial_forward(*[x.to(dev) for x in inp[:5]], w1, w2, scale, kb, vb, flags=flags)
+
+
+def oracle_rows(inp, w1, w2, rows, scale=None, kb=0.0, vb=0.0, dtype=torch.float64):
+    return orc.forward_windowed(*[x.to(dtype) for x in inp[:5]], w1, w2, scale, kb, vb, rows=rows,
+                                compute_dtype=dtype)
+
+
+SMALL = [  # B, N, H, D, w1, w2, k2_bias, v2_bias
+    (1, 64, 1, 64, 16, 8, 0.0, 0.0),
+    (2, 100, 2, 128, 40, 5, 0.0, 0.0),        # N not a multiple of the tile
+    (1, 256, 2, 64, 512, 32, 0.0, 0.0),       # windows wider than the sequence
+    (1, 200, 1, 128, 0, 0, 0.0, 0.0),         # single-triple windows
+    (1, 130, 2, 64, 33, 1, 0.1, 0.2),
+    (1, 96, 1, 128, 7, 64, -0.1, -0.2),       # K' window wider than the K window
+    (2, 160, 3, 128, 64, 32, 1.0, 0.5),
+    (1, 33, 1, 64, 31, 32, 0.0, 0.0),
+    (1, 1, 1, 64, 4, 4, 0.0, 0.0),
+]
+
+
+@pytest.mark.parametrize("case", SMALL)
+def test_small_shapes_vs_oracle(case):
+    B, N, H, D, w1, w2, kb, vb = case
+    inp = make_inputs(B, N, H, D, seed=N + D + w1, dtype=torch.bfloat16, with_dout=False)
+    out, lse = fwd(inp, w1, w2, None, kb, vb)
+    want, want_lse = oracle_rows(inp, w1, w2, None, None, kb, vb)
+    assert_close_rel(out, want, BF16_TOL, "out")
+    assert_close_rel(lse, want_lse, BF16_TOL, "lse")
+
+
+def test_auto_dispatch_takes_mfma_for_bf16_d64_d128():
+    from simplical_attn_amd import _lib
+    lib = _lib.load()
+    assert lib.sa2_uses_mfma(2, 2048, 8, 64, 512, 32, _lib.SA2_BF16) == 1
+    assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_BF16) == 1
+    assert lib.sa2_uses_mfma(1, 128, 2, 64, 32, 16, _lib.SA2_F32) == 0
+    assert lib.sa2_uses_mfma(1, 128, 2, 32, 32, 16, _lib.SA2_BF16) == 0
+    inp = make_inputs(1, 96, 2, 64, seed=1, dtype=torch.bfloat16, with_dout=False)
+    a = fwd(inp, 20, 6, flags=0)
+    b = fwd(inp, 20, 6, flags=MFMA)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_config2_forward():
+    """BASELINE config 2: bf16, B2 H8 N2048 D64, w 512/32, seed 1."""
+    inp = make_inputs(2, 2048, 8, 64, seed=1, dtype=torch.bfloat16, with_dout=False)
+    out, lse = fwd(inp, 512, 32)
+    for rows in ((0, 96), (480, 576), (1990, 2048)):
+        want, want_lse = oracle_rows(inp, 512, 32, rows, dtype=torch.float32)
+        assert_close_rel(out[:, rows[0]:rows[1]], want, BF16_TOL, "out rows %s" % (rows,))
+        assert_close_rel(lse[:, :, rows[0]:rows[1]], want_lse, BF16_TOL, "lse rows %s" % (rows,))
+    ref, ref_lse = fwd(inp, 512, 32, flags=GENERIC)
+    assert_close_rel(out, ref.float().cpu(), BF16_TOL, "out vs generic kernel")
+    assert_close_rel(lse, ref_lse.cpu(), BF16_TOL, "lse vs generic kernel")
+
+
+def test_config4_forward_headline_shape():
+    """BASELINE config 4: bf16, B1 H16 N8192 D128, w 512/32, seed 3; oracle on
+    row ranges (start, the block straddling i = w1, end), generic kernel on all rows."""
+    inp = make_inputs(1, 8192, 16, 128, seed=3, dtype=torch.bfloat16, with_dout=False)
+    out, lse = fwd(inp, 512, 32)
+    for rows in ((0, 40), (500, 540), (8160, 8192)):
+        want, want_lse = oracle_rows(inp, 512, 32, rows, dtype=torch.float32)
+        assert_close_rel(out[:, rows[0]:rows[1]], want, BF16_TOL, "out rows %s" % (rows,))
+        assert_close_rel(lse[:, :, rows[0]:rows[1]], want_lse, BF16_TOL, "lse rows %s" % (rows,))
+    ref, ref_lse = fwd(inp, 512, 32, flags=GENERIC)
+    assert_close_rel(out, ref.float().cpu(), BF16_TOL, "out vs generic kernel")
+    assert_close_rel(lse, ref_lse.cpu(), BF16_TOL, "lse vs generic kernel")
+
+
+def test_extreme_and_zero_inputs():
+    dev = torch.device("cuda:0")
+    import simplical_attn_amd as sa
+    t = torch.full((1, 64, 2, 64), 10.0, device=dev, dtype=torch.bfloat16)
+    out, lse = sa.simplicial_forward(t, t, t, t, t, 8, 8, flags=MFMA)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert torch.allclose(out.float(), torch.full_like(out, 100.0).float(), rtol=1e-2)
+    z = torch.zeros_like(t)
+    out, lse = sa.simplicial_forward(z, z, z, z, z, 8, 8, flags=MFMA)
+    assert torch.equal(out, torch.zeros_like(out))
+    want = torch.tensor([math.log((min(i, 8) + 1) ** 2 + 1e-8) for i in range(64)])
+    assert torch.allclose(lse[0, 0].cpu(), want.float(), rtol=1e-5)
+
+
+def test_deterministic():
+    inp = make_inputs(2, 300, 2, 128, seed=42, dtype=torch.bfloat16, with_dout=False)
+    a = fwd(inp, 100, 20)
+    b = fwd(inp, 100, 20)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
