@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the 2-simplicial attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5]
+
+A step is one forward + backward pass of the operator over one batch of
+synthetic input that is already resident in HBM (iid normal, seeded, bf16).
+The default workload is the headline configuration: bf16, B=1 H=16 N=8192 D=128,
+w1=512 w2=32.  Prints ONE JSON line:
+
+  metric/value   forward+backward algorithmic TFLOP/s: 16*D*T flops per step,
+                 T = number of valid (i,j,k) triples (matmul flops only, 2 per
+                 MAC: 4*D*T forward, 12*D*T backward)
+  roofline       the kernel that dominates the step, against the bf16 dense MFMA
+                 peak (achieved = that kernel's algorithmic flops / its duration,
+                 measured here with events on the launch stream)
+  kernels        the same for every kernel group of the step, plus HBM GB/s
+  cpu_baseline   the CPU oracle (a port of the reference's PyTorch loop) timed on
+                 this host on a bounded sample of the same workload
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
+PEAK_FP32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, N, H, D, w1, w2, seed, qk_std)
+    "c2": (2, 2048, 8, 64, 512, 32, 1, 1.0),
+    "c4": (1, 8192, 16, 128, 512, 32, 3, 1.0),
+    "c5": (1, 32768, 8, 128, 1024, 64, 4, 0.5),
+}
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
+# scaled by the same counters on a plain copy kernel; None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def count_triples(B, N, H, w1, w2):
+    return B * H * sum((min(i, w1) + 1) * (min(i, w2) + 1) for i in range(N))
+
+
+def make_inputs(B, N, H, D, seed, qk_std, device):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for t in range(6):
+        x = torch.randn(B, N, H, D, generator=g, dtype=torch.float32)
+        if t < 3:
+            x = x * qk_std
+        out.append(x.to(torch.bfloat16).to(device))
+    return out
+
+
+def time_gpu(fn, steps, warmup):
+    """Average milliseconds per call, events on the current (launch) stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline(name, cfg, budget_rows):
+    """Times the CPU oracle forward + autograd on `budget_rows` steady-state
+    query rows of the workload (all batches and heads) and scales by the triple
+    count.  Returns the JSON object."""
+    from oracle import simplicial_oracle as orc
+    B, N, H, D, w1, w2, seed, qk_std = cfg
+    g = torch.Generator().manual_seed(seed)
+    tens = []
+    for t in range(6):
+        x = torch.randn(B, N, H, D, generator=g, dtype=torch.float32)
+        if t < 3:
+            x = x * qk_std
+        tens.append(x.to(torch.bfloat16).float())
+    r0 = min(N - budget_rows, max(w1, w2) + 64)
+    r0 = max(r0, 0)
+    r1 = min(N, r0 + budget_rows)
+    t0 = time.perf_counter()
+    orc.grads_windowed(*tens[:5], tens[5][:, r0:r1], w1, w2, rows=(r0, r1), chunk=16, compute_dtype=torch.float32)
+    dt = time.perf_counter() - t0
+    t_rows = B * H * sum((min(i, w1) + 1) * (min(i, w2) + 1) for i in range(r0, r1))
+    flops = 16.0 * D * t_rows
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": "oracle forward+autograd (fp32, vectorised restatement of reference.py) on query rows "
+                  "[%d,%d) of workload %s, all %d heads; %.1f s; scaled by triple count" % (r0, r1, name, B * H, dt),
+        "seconds": dt, "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=2560)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (heads are independent and would "
+              "shard with no communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    import simplical_attn_amd as sa
+    from simplical_attn_amd import _lib
+    lib = _lib.load()
+
+    cfg = WORKLOADS[args.workload]
+    B, N, H, D, w1, w2, seed, qk_std = cfg
+    dev = torch.device("cuda:0")
+    props = torch.cuda.get_device_properties(0)
+    q, k1, k2, v1, v2, dout = make_inputs(B, N, H, D, seed, qk_std, dev)
+    T = count_triples(B, N, H, w1, w2)
+    fwd_flops, bwd_flops = 4.0 * D * T, 12.0 * D * T
+    E = B * N * H * D
+    fwd_bytes = 6 * E * 2 + 4 * B * H * N                  # read q,k1,k2,v1,v2; write O, LSE
+    bwd_bytes = 12 * E * 2 + 12 * B * H * N                # read 5 inputs, O, dO; write 5 grads; LSE, D
+
+    leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+    attn = sa.TwoSimplicialAttention(D, w1, w2)
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        out = attn(*leaves)
+        out.backward(dout)
+
+    # ---- the timed region: K full steps --------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+
+    # ---- per-kernel-group durations (same stream, events) -------------------
+    out, lse = sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2)
+    ksteps = max(5, args.steps)
+    fwd_ms = time_gpu(lambda: sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2), ksteps, 2)
+    rowdot_ms = time_gpu(lambda: sa.compute_D_kernel(dout, out), ksteps, 2)
+    bwd_all_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2), ksteps, 2)
+    bwd_k1_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2,
+                                                        needs=(False, True, False, True, False)), ksteps, 2) - rowdot_ms
+    bwd_rest_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2,
+                                                          needs=(True, False, True, False, True)), ksteps, 2) - rowdot_ms
+    mfma = bool(lib.sa2_uses_mfma(B, N, H, D, w1, w2, _lib.SA2_BF16))
+    kernels = {
+        "forward": {"ms": fwd_ms, "tflops": fwd_flops / fwd_ms / 1e9, "hbm_gbs": fwd_bytes / fwd_ms / 1e6},
+        "backward": {"ms": bwd_all_ms, "tflops": bwd_flops / bwd_all_ms / 1e9, "hbm_gbs": bwd_bytes / bwd_all_ms / 1e6},
+        "backward_dk_dv": {"ms": bwd_k1_ms},
+        "backward_dq_dk2_dv2": {"ms": bwd_rest_ms},
+        "rowdot": {"ms": rowdot_ms, "hbm_gbs": (4 * E + 4 * B * H * N) / rowdot_ms / 1e6},
+    }
+    for k in ("forward", "backward"):
+        kernels[k]["frac_bf16_peak"] = kernels[k]["tflops"] / PEAK_BF16_TFLOPS
+
+    # The forward kernel is one launch; its duration is the forward call's.
+    dominant = "forward" if fwd_ms >= bwd_all_ms else "backward"
+    roofline = {
+        "bound": "mfma", "kernel": "mfma_fwd_kernel<%d>" % D if dominant == "forward" else "backward kernels (sum)",
+        "achieved": kernels[dominant]["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+        "frac": kernels[dominant]["tflops"] / PEAK_BF16_TFLOPS,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dominant)),
+        "algorithmic_flops_per_launch": fwd_flops if dominant == "forward" else bwd_flops,
+        "avg_ms": kernels[dominant]["ms"],
+    }
+    roofline_fwd = {
+        "bound": "mfma", "kernel": "mfma_fwd_kernel<%d>" % D, "achieved": kernels["forward"]["tflops"],
+        "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": kernels["forward"]["frac_bf16_peak"],
+        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "forward")),
+        "hbm_gbs": kernels["forward"]["hbm_gbs"], "hbm_frac": kernels["forward"]["hbm_gbs"] / PEAK_HBM_GBS,
+    }
+
+    line = {
+        "metric": "fwd+bwd TFLOP/s & %% bf16 MFMA peak, N=%d D=%d w1=%d w2=%d" % (N, D, w1, w2),
+        "value": (fwd_flops + bwd_flops) / ms_per_step / 1e9,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "wall_ms_per_step": wall_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%s: bf16 fwd+bwd B=%d H=%d N=%d D=%d w1=%d w2=%d scale=1/sqrt(D)" % (
+                       args.workload, B, H, N, D, w1, w2),
+                   "triples": T, "flops_fwd": fwd_flops, "flops_bwd": bwd_flops,
+                   "mfma_kernels": mfma, "device": props.name, "cus": props.multi_processor_count,
+                   "clock_mhz": props.clock_rate / 1e3 if hasattr(props, "clock_rate") else None},
+        "frac_bf16_peak": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
+        "roofline": roofline,
+        "roofline_forward": roofline_fwd,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_rows)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

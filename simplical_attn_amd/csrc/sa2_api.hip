@@ -8,8 +8,6 @@ using namespace sa2;
 
 namespace {
 
-int elem_size(int dtype) { return dtype == SA2_F32 ? 4 : 2; }
-
 bool valid_dtype(int dtype) { return dtype == SA2_F32 || dtype == SA2_BF16 || dtype == SA2_F16; }
 
 int check_dims(int B, int N, int H, int D, int w1, int w2, int dtype, int window_inclusive) {
@@ -52,7 +50,9 @@ size_t dsum_bytes(int B, int N, int H) { return align_up((size_t)B * H * N * siz
 bool pick_mfma(const Problem& p, int dtype, unsigned flags, bool backward, int* status) {
     *status = SA2_OK;
     if (flags & SA2_FLAG_FORCE_GENERIC) return false;
-    const bool ok = mfma_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype) && mfma_layout_ok(p, backward);
+    const bool ok = (backward ? mfma_bwd_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)
+                              : mfma_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)) &&
+                    mfma_layout_ok(p, backward);
     if (!ok && (flags & SA2_FLAG_FORCE_MFMA)) *status = SA2_ERR_UNSUPPORTED;
     return ok;
 }
@@ -116,7 +116,7 @@ int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, c
 size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int dtype, unsigned flags) {
     if (check_dims(B, N, H, D, w1, w2, dtype, 1) != SA2_OK) return 0;
     size_t scratch = generic_bwd_scratch_bytes(B, N, H, D, w1, w2);
-    if (!(flags & SA2_FLAG_FORCE_GENERIC) && mfma_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype)) {
+    if (!(flags & SA2_FLAG_FORCE_GENERIC) && mfma_bwd_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype)) {
         const size_t m = mfma_bwd_scratch_bytes(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N));
         if (m > scratch) scratch = m;
     }

@@ -73,6 +73,7 @@ int launch_generic_bwd(const Problem& p, int dtype, hipStream_t st);
 size_t generic_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 
 bool mfma_supported(int B, int N, int H, int D, int w1, int w2, int dtype);
+bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype);
 bool mfma_layout_ok(const Problem& p, bool backward);
 int launch_mfma_fwd(const Problem& p, hipStream_t st);
 int launch_mfma_bwd(const Problem& p, hipStream_t st);

@@ -51,14 +51,37 @@ struct Cfg {
     static constexpr int VPASS = NDP / 32;                  // 4-row groups per thread per tile
     static constexpr int OS = D + 4;                        // merge buffer row stride (fp32)
     static constexpr int MERGE_FLOATS = 4 * (BQ * OS + 2 * BQ);
-    static constexpr size_t LDS_BYTES =
-        (2 * STAGE * 2 > MERGE_FLOATS * 4) ? (size_t)2 * STAGE * 2 : (size_t)MERGE_FLOATS * 4;
+    static constexpr size_t STAGE_BYTES = (size_t)2 * STAGE * 2;          // two staging buffers
+    static constexpr size_t LDS_BYTES = STAGE_BYTES + (size_t)MERGE_FLOATS * 4;
 };
 
 __device__ __forceinline__ float bf16_lo(uint32_t x) { return __uint_as_float(x << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float other_half(float x) { return __shfl_xor(x, 32); }
+
+// Exchange between lane l and lane l^32 (one VALU op): returns the partner's value.
+__device__ __forceinline__ float other_half(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    // r[0] holds the low half's value in every lane, r[1] the high half's
+    return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+}
+
+// acc *= alpha for an MFMA accumulator that lives in AGPRs, without asking the
+// register allocator for a VGPR copy of the tuple (it would place that copy on
+// the hot path).  Used only on the rare rescale path; the s_nop before the
+// first read covers the MFMA-write -> VALU-read distance, the one after the
+// last write the VALU-write -> MFMA-read distance.
+__device__ __forceinline__ void scale_acc(floatx16& acc, float alpha) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        float x = acc[v], t;
+        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                     : "+a"(x), "=&v"(t)
+                     : "v"(alpha));
+        acc[v] = x;
+    }
+}
 
 template <int D>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
@@ -150,22 +173,19 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     };
 
     // ---- per-wavefront state -------------------------------------------------
-    floatx16 oacc[C::DT];
+    // The query accumulators O (fp32, unnormalised, relative to Mrun) live in
+    // LDS behind the staging buffers: they are touched once per unit, and the
+    // registers they would take are what keeps the sweep free of AGPR copies.
+    float* fm = (float*)(smem_raw + C::STAGE_BYTES);
+    float* Om = fm + wave * (BQ * C::OS + 2 * BQ);
+    float* Mm = Om + BQ * C::OS;
+    float* Lm = Mm + BQ;
 #pragma unroll
     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[dt][v] = 0.f;
+        for (int g4 = 0; g4 < 4; ++g4)
+            *(float4*)(Om + ln * C::OS + dt * 32 + 8 * g4 + 4 * hf) = make_float4(0.f, 0.f, 0.f, 0.f);
     float Mrun = -INFINITY, Lrun = 0.f;
-
-    bf16x8 qf[2][C::DK];
-    floatx16 racc[2][C::DT];
-    float m[2], l[2];
-    int delta[2];
-    bool unit_ok[2];
-    delta[0] = delta[1] = 0;
-    unit_ok[0] = unit_ok[1] = false;
-    m[0] = m[1] = -INFINITY;
-    l[0] = l[1] = 0.f;
 
     const float qscale = p.scale * LOG2E;
 
@@ -174,48 +194,56 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     if (total_steps > 1) load_tile(jt_lo + (1 % nt));
     __syncthreads();
 
-    int s = 0, round = 0;
-    for (int g = 0; g < total_steps; ++g) {
-        const int jt = jt_lo + s;
-        const int j0 = jt * TJ;
-        if (s == 0) {
-            // new pair of units: form Q~ operands, reset the running softmax
-            const int pair = round * 4 + wave;
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                delta[u] = 2 * pair + u;
-                unit_ok[u] = delta[u] < n_units;
-                m[u] = -INFINITY;
-                l[u] = 0.f;
-#pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) racc[u][dt][v] = 0.f;
-                int k = ic - delta[u];
-                k = k > 0 ? k : 0;
-#pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) {
-                    bf16x8 r;
-                    if (unit_ok[u]) {
-                        const uint4 qa = *(const uint4*)(qp + (int64_t)ic * p.q.sn + kk * 16 + hf * 8);
-                        const uint4 kb = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + kk * 16 + hf * 8);
-                        const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
-                        const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) {
-                            r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
-                            r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
-                        }
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 8; ++t) r[t] = (__bf16)0.f;
-                    }
-                    qf[u][kk] = r;
-                }
+    int g = 0;
+    for (int round = 0; round < nrounds; ++round) {
+        const int pair = round * 4 + wave;
+        const int delta0 = 2 * pair, delta1 = 2 * pair + 1;
+        const bool ok0 = delta0 < n_units, ok1 = delta1 < n_units;
+
+        if (!ok0) {
+            // nothing to compute this round: keep the staging pipeline moving
+            for (int s = 0; s < nt; ++s, ++g) {
+                if (g + 1 < total_steps) store_tile((g + 1) & 1);
+                if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
+                __syncthreads();
             }
+            continue;
         }
 
-        if (unit_ok[0]) {
+        // ---- new pair of units: Q~ operands, fresh running softmax ----------
+        bf16x8 qf[2][C::DK];
+        floatx16 racc[2][C::DT];
+        float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) racc[u][dt][v] = 0.f;
+            int k = ic - (u ? delta1 : delta0);
+            k = k > 0 ? k : 0;
+#pragma unroll
+            for (int kk = 0; kk < C::DK; ++kk) {
+                const uint4 qa = *(const uint4*)(qp + (int64_t)ic * p.q.sn + kk * 16 + hf * 8);
+                const uint4 kb = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + kk * 16 + hf * 8);
+                const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
+                const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
+                bf16x8 r;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
+                    r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
+                }
+                qf[u][kk] = r;
+            }
+        }
+        const bool rows_full0 = i0 >= delta0 && i0 + BQ - 1 < N;
+        const bool rows_full1 = ok1 && i0 >= delta1 && i0 + BQ - 1 < N;
+        const bool row_ok0 = i < N && i >= delta0;
+        const bool row_ok1 = ok1 && i < N && i >= delta1;
+
+        for (int s = 0; s < nt; ++s, ++g) {
+            const int j0 = (jt_lo + s) * TJ;
             const uint16_t* Ks = smem + (g & 1) * C::STAGE;
             const uint16_t* Vt = Ks + C::K_ELEMS;
             // S^T tiles: rows = keys of the tile, columns = expanded rows
@@ -230,46 +258,49 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                 sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[0][kk], sacc[0], 0, 0, 0);
                 sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[1][kk], sacc[1], 0, 0, 0);
             }
-            const bool interior = (j0 + TJ - 1 <= i0) && (j0 >= i0 + BQ - 1 - w1) && (i0 + BQ - 1 < N);
+            const bool interior = (j0 + TJ - 1 <= i0) && (j0 >= i0 + BQ - 1 - w1);
             bf16x8 pb[2][2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                if (!(interior && unit_ok[u] && i0 >= delta[u])) {
+                float pv[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) pv[v] = sacc[u][v];
+                if (__builtin_expect(!(interior && (u ? rows_full1 : rows_full0)), 0)) {
                     // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
-                    const bool row_ok = unit_ok[u] && i < N && i >= delta[u];
+                    const bool row_ok = u ? row_ok1 : row_ok0;
                     const int hi = i - j0 - 4 * hf, lo = hi - w1;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int c = 8 * (v >> 2) + (v & 3);
-                        sacc[u][v] = (row_ok && c <= hi && c >= lo) ? sacc[u][v] : -INFINITY;
+                        pv[v] = (row_ok && c <= hi && c >= lo) ? pv[v] : -INFINITY;
                     }
                 }
-                float mx = sacc[u][0];
+                float mx = fmaxf(pv[0], pv[1]);
 #pragma unroll
-                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, sacc[u][v]);
+                for (int v = 2; v < 16; ++v) mx = fmaxf(mx, pv[v]);
                 mx = fmaxf(mx, other_half(mx));
                 // Lazy reference point: move it only when the maximum grows by more
                 // than 2^RESCALE_LOG2, so the accumulator rescale is rare; weights
                 // stay below 2^RESCALE_LOG2 and every later formula only needs m to
                 // be a common reference, not the exact maximum.
-                const float m_new = (mx > m[u] + RESCALE_LOG2) ? mx : m[u];
-                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                const float alpha = fast_exp2(m[u] - m_use);
-                m[u] = m_new;
+                if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[u] + RESCALE_LOG2) != 0, 0)) {
+                    const float m_new = (mx > m[u] + RESCALE_LOG2) ? mx : m[u];
+                    const float alpha = fast_exp2(m[u] - ((m_new == -INFINITY) ? 0.f : m_new));
+                    m[u] = m_new;
+                    l[u] *= alpha;
+                    asm volatile("s_nop 15\n\ts_nop 15");
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt) scale_acc(racc[u][dt], alpha);
+                    asm volatile("s_nop 4");
+                }
+                const float m_use = (m[u] == -INFINITY) ? 0.f : m[u];
                 float rs = 0.f;
-                float pv[16];
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    pv[v] = fast_exp2(sacc[u][v] - m_use);
+                    pv[v] = fast_exp2(pv[v] - m_use);
                     rs += pv[v];
                 }
-                l[u] = l[u] * alpha + rs;
-                if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) racc[u][dt][v] *= alpha;
-                }
+                l[u] += rs;
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
@@ -285,61 +316,53 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                     racc[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][ks], racc[1][dt], 0, 0, 0);
                 }
 
-            if (s == nt - 1) {
-                // fold the finished units into the query accumulators
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    if (!unit_ok[u]) continue;
-                    const float lt = l[u] + other_half(l[u]);
-                    const float Mn = fmaxf(Mrun, m[u]);
-                    const float Muse = (Mn == -INFINITY) ? 0.f : Mn;
-                    const float a = fast_exp2(Mrun - Muse), bb = fast_exp2(m[u] - Muse);
-                    Lrun = Lrun * a + lt * bb;
-                    Mrun = Mn;
-                    int k = ic - delta[u];
-                    k = k > 0 ? k : 0;
-                    const uint16_t* vrow = v2p + (int64_t)k * p.v2.sn + 4 * hf;
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                        for (int g4 = 0; g4 < 4; ++g4) {
-                            const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
-                            const float f0 = bf16_lo(x.x) + p.v2_bias, f1 = bf16_hi(x.x) + p.v2_bias;
-                            const float f2 = bf16_lo(x.y) + p.v2_bias, f3 = bf16_hi(x.y) + p.v2_bias;
-                            oacc[dt][4 * g4 + 0] = oacc[dt][4 * g4 + 0] * a + bb * racc[u][dt][4 * g4 + 0] * f0;
-                            oacc[dt][4 * g4 + 1] = oacc[dt][4 * g4 + 1] * a + bb * racc[u][dt][4 * g4 + 1] * f1;
-                            oacc[dt][4 * g4 + 2] = oacc[dt][4 * g4 + 2] * a + bb * racc[u][dt][4 * g4 + 2] * f2;
-                            oacc[dt][4 * g4 + 3] = oacc[dt][4 * g4 + 3] * a + bb * racc[u][dt][4 * g4 + 3] * f3;
-                        }
-                }
-            }
+            if (g + 1 < total_steps) store_tile((g + 1) & 1);
+            if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
+            __syncthreads();
         }
 
-        if (g + 1 < total_steps) store_tile((g + 1) & 1);
-        if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
-        __syncthreads();
-        if (++s == nt) {
-            s = 0;
-            ++round;
+        // ---- fold the finished units into the query accumulators ------------
+        float a_all = 1.f, bb[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const float lt = l[u] + other_half(l[u]);
+            const float Mn = fmaxf(Mrun, m[u]);
+            const float Muse = (Mn == -INFINITY) ? 0.f : Mn;
+            const float a = fast_exp2(Mrun - Muse);
+            bb[u] = fast_exp2(m[u] - Muse);
+            // unit 0's factor must also shrink by unit 1's rescale of the accumulator
+            if (u == 1) bb[0] *= a;
+            a_all *= a;
+            Lrun = Lrun * a + lt * bb[u];
+            Mrun = Mn;
         }
+        int kr0 = ic - delta0, kr1 = ic - delta1;
+        kr0 = kr0 > 0 ? kr0 : 0;
+        kr1 = kr1 > 0 ? kr1 : 0;
+        const uint16_t* vrow0 = v2p + (int64_t)kr0 * p.v2.sn + 4 * hf;
+        const uint16_t* vrow1 = v2p + (int64_t)kr1 * p.v2.sn + 4 * hf;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const uint2 x0 = *(const uint2*)(vrow0 + dt * 32 + 8 * g4);
+                const uint2 x1 = *(const uint2*)(vrow1 + dt * 32 + 8 * g4);
+                float* op = Om + ln * C::OS + dt * 32 + 8 * g4 + 4 * hf;
+                float4 o = *(float4*)op;
+                const float b0 = bb[0], b1 = bb[1];
+                o.x = o.x * a_all + b0 * racc[0][dt][4 * g4 + 0] * (bf16_lo(x0.x) + p.v2_bias) +
+                      b1 * racc[1][dt][4 * g4 + 0] * (bf16_lo(x1.x) + p.v2_bias);
+                o.y = o.y * a_all + b0 * racc[0][dt][4 * g4 + 1] * (bf16_hi(x0.x) + p.v2_bias) +
+                      b1 * racc[1][dt][4 * g4 + 1] * (bf16_hi(x1.x) + p.v2_bias);
+                o.z = o.z * a_all + b0 * racc[0][dt][4 * g4 + 2] * (bf16_lo(x0.y) + p.v2_bias) +
+                      b1 * racc[1][dt][4 * g4 + 2] * (bf16_lo(x1.y) + p.v2_bias);
+                o.w = o.w * a_all + b0 * racc[0][dt][4 * g4 + 3] * (bf16_hi(x0.y) + p.v2_bias) +
+                      b1 * racc[1][dt][4 * g4 + 3] * (bf16_hi(x1.y) + p.v2_bias);
+                *(float4*)op = o;
+            }
     }
 
     // ---- merge the four wavefronts' partial (M, L, O) through LDS ------------
-    float* fm = (float*)smem_raw;
-    float* Om = fm + wave * (BQ * C::OS + 2 * BQ);
-    float* Mm = Om + BQ * C::OS;
-    float* Lm = Mm + BQ;
-#pragma unroll
-    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            float4 x;
-            x.x = oacc[dt][4 * g4 + 0];
-            x.y = oacc[dt][4 * g4 + 1];
-            x.z = oacc[dt][4 * g4 + 2];
-            x.w = oacc[dt][4 * g4 + 3];
-            *(float4*)(Om + ln * C::OS + dt * 32 + 8 * g4 + 4 * hf) = x;
-        }
     if (hf == 0) {
         Mm[ln] = Mrun;
         Lm[ln] = Lrun;
