@@ -20,22 +20,10 @@
 // lives in one lane (pair): row maxima and sums are in-lane reductions plus one
 // exchange with lane^32, and exp2(S^T) is already laid out as the B operand of
 // R^T = V^T . P^T.
-#include "sa2_common.h"
+#include "sa2_mfma_common.h"
 
 namespace sa2 {
 namespace {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(16))) float floatx16;
-
-constexpr int BQ = 32;       // queries per workgroup
-constexpr int TJ = 32;       // keys per LDS tile
-constexpr int NTHREADS = 256;
-constexpr float RESCALE_LOG2 = 8.0f;
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LN2 = 0.6931471805599453f;
-constexpr float LOG2_EPS = -26.575424759098897f;   // log2(1e-8)
-constexpr float LN_EPS = -18.420680743952367f;     // ln(1e-8)
 
 template <int D>
 struct Cfg {
@@ -54,34 +42,6 @@ struct Cfg {
     static constexpr size_t STAGE_BYTES = (size_t)2 * STAGE * 2;          // two staging buffers
     static constexpr size_t LDS_BYTES = STAGE_BYTES + (size_t)MERGE_FLOATS * 4;
 };
-
-__device__ __forceinline__ float bf16_lo(uint32_t x) { return __uint_as_float(x << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// Exchange between lane l and lane l^32 (one VALU op): returns the partner's value.
-__device__ __forceinline__ float other_half(float x) {
-    const unsigned u = __float_as_uint(x);
-    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    // r[0] holds the low half's value in every lane, r[1] the high half's
-    return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
-}
-
-// acc *= alpha for an MFMA accumulator that lives in AGPRs, without asking the
-// register allocator for a VGPR copy of the tuple (it would place that copy on
-// the hot path).  Used only on the rare rescale path; the s_nop before the
-// first read covers the MFMA-write -> VALU-read distance, the one after the
-// last write the VALU-write -> MFMA-read distance.
-__device__ __forceinline__ void scale_acc(floatx16& acc, float alpha) {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        float x = acc[v], t;
-        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
-                     : "+a"(x), "=&v"(t)
-                     : "v"(alpha));
-        acc[v] = x;
-    }
-}
 
 template <int D>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
