@@ -320,6 +320,271 @@ __global__ __launch_bounds__(256) void mfma_bwd_finalize_kernel(Problem p, const
     }
 }
 
+// ========================================================== column kernel ====
+constexpr int CJ = 128;      // K rows per workgroup (32 per wavefront)
+
+template <int D>
+struct ColCfg {
+    static constexpr int DK = D / 16;
+    static constexpr int DT = D / 32;
+    static constexpr int KS = D + 8;           // row-major unit tile row stride (bf16)
+    static constexpr int VS = BQ + 8;          // transposed unit tile row stride (bf16)
+    static constexpr int RM_ELEMS = BQ * KS;
+    static constexpr int TR_ELEMS = D * VS;
+    static constexpr int UNIT = 2 * RM_ELEMS + 2 * TR_ELEMS;    // Q~, dO~ row-major; Q~^T, dO~^T
+    static constexpr int RAW_Q = BQ * D;                        // q and dO rows of the query block
+    static constexpr int RAW_K = 2 * BQ * D;                    // 64 rows of k2 / v2 per delta chunk
+    static constexpr int RAW = 2 * RAW_Q + 2 * RAW_K;
+    static constexpr int NCP = D / 2;                           // column pairs
+    static constexpr int COMBOS = 8 * NCP / NTHREADS;           // (4-row group, column pair) items per thread
+    static constexpr size_t LDS_BYTES = (size_t)(2 * UNIT + RAW) * 2 + 2 * BQ * sizeof(float);
+};
+
+template <int D>
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void mfma_bwd_col_kernel(Problem p, int njb, int total) {
+    using C = ColCfg<D>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    uint16_t* units = (uint16_t*)smem_raw;                 // two formed units
+    uint16_t* q_s = units + 2 * C::UNIT;
+    uint16_t* do_s = q_s + C::RAW_Q;
+    uint16_t* k2_s = do_s + C::RAW_Q;
+    uint16_t* v2_s = k2_s + C::RAW_K;
+    float* lse_s = (float*)(v2_s + C::RAW_K);
+    float* dsum_s = lse_s + BQ;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, ln = lane & 31, hf = lane >> 5;
+
+    int pid = blockIdx.x;
+    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    const int bh = pid / njb, jb = pid - bh * njb;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int N = p.N, w1 = p.w1, w2 = p.w2;
+    const int j0 = jb * CJ;
+    const int jw = j0 + 32 * wave;               // this wavefront's K rows: jw .. jw+31
+    const int j = jw + ln;
+    const int jc = j < N ? j : N - 1;
+
+    const uint16_t* qp = (const uint16_t*)p.q.p + p.q.off(b, 0, h);
+    const uint16_t* k1p = (const uint16_t*)p.k1.p + p.k1.off(b, 0, h);
+    const uint16_t* k2p = (const uint16_t*)p.k2.p + p.k2.off(b, 0, h);
+    const uint16_t* v1p = (const uint16_t*)p.v1.p + p.v1.off(b, 0, h);
+    const uint16_t* v2p = (const uint16_t*)p.v2.p + p.v2.off(b, 0, h);
+    const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
+
+    // K and V rows of this wavefront as resident MFMA B operands (column = K row)
+    bf16x8 kfr[C::DK], vfr[C::DK];
+#pragma unroll
+    for (int kk = 0; kk < C::DK; ++kk) {
+        kfr[kk] = *(const bf16x8*)(k1p + (int64_t)jc * p.k1.sn + kk * 16 + hf * 8);
+        vfr[kk] = *(const bf16x8*)(v1p + (int64_t)jc * p.v1.sn + kk * 16 + hf * 8);
+    }
+    floatx16 dkacc[C::DT], dvacc[C::DT];
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dkacc[dt][v] = dvacc[dt][v] = 0.f;
+
+    const float qscale = p.scale * LOG2E;
+    const int j_last = (j0 + CJ - 1 < N ? j0 + CJ - 1 : N - 1);
+    const int i_max = (int)((int64_t)j_last + w1 < N - 1 ? j_last + w1 : N - 1);
+    const int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+
+    for (int ib = ib_lo; ib <= ib_hi; ++ib) {
+        const int i0 = ib * BQ;
+        const int i_last = (i0 + BQ - 1 < N ? i0 + BQ - 1 : N - 1);
+        const int n_units = (w2 < i_last ? w2 : i_last) + 1;
+        // does this wavefront's K tile see any query of the block?
+        const bool touches = (i0 + BQ - 1 >= jw) && ((int64_t)i0 <= (int64_t)jw + 31 + w1) && jw < N;
+        float lse2r[16], dsumr[16];
+
+        for (int dc = 0; dc < n_units; dc += BQ) {
+            const int ndl = (n_units - dc < BQ ? n_units - dc : BQ);
+            const int kbase = i0 - dc - BQ;         // k2_s / v2_s row 0
+            __syncthreads();
+            // ---- raw rows: q, dO of the block (once) and 64 rows of k2, v2 ------
+            if (dc == 0) {
+#pragma unroll
+                for (int u = 0; u < BQ * D / 8 / NTHREADS; ++u) {
+                    const int c = tid + NTHREADS * u;
+                    const int row = c / (D / 8), col = c - row * (D / 8);
+                    int i = i0 + row;
+                    i = i < N ? i : N - 1;
+                    *(uint4*)(q_s + row * D + col * 8) = *(const uint4*)(qp + (int64_t)i * p.q.sn + col * 8);
+                    *(uint4*)(do_s + row * D + col * 8) = *(const uint4*)(dop + (int64_t)i * p.dout.sn + col * 8);
+                }
+                if (tid < BQ) {
+                    int i = i0 + tid;
+                    i = i < N ? i : N - 1;
+                    lse_s[tid] = p.lse[(int64_t)bh * N + i] * LOG2E;
+                    dsum_s[tid] = p.dsum[(int64_t)bh * N + i];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 2 * BQ * D / 8 / NTHREADS; ++u) {
+                const int c = tid + NTHREADS * u;
+                const int row = c / (D / 8), col = c - row * (D / 8);
+                int k = kbase + row;
+                k = k < 0 ? 0 : (k < N ? k : N - 1);
+                *(uint4*)(k2_s + row * D + col * 8) = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + col * 8);
+                *(uint4*)(v2_s + row * D + col * 8) = *(const uint4*)(v2p + (int64_t)k * p.v2.sn + col * 8);
+            }
+            __syncthreads();
+            if (dc == 0) {
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const float4 a = *(const float4*)(lse_s + 8 * g4 + 4 * hf);
+                    const float4 c = *(const float4*)(dsum_s + 8 * g4 + 4 * hf);
+                    lse2r[4 * g4] = a.x; lse2r[4 * g4 + 1] = a.y; lse2r[4 * g4 + 2] = a.z; lse2r[4 * g4 + 3] = a.w;
+                    dsumr[4 * g4] = c.x; dsumr[4 * g4 + 1] = c.y; dsumr[4 * g4 + 2] = c.z; dsumr[4 * g4 + 3] = c.w;
+                }
+            }
+
+            // Form the expanded rows of one delta in all four layouts.
+            auto form = [&](int delta, int buf) {
+                uint16_t* Qr = units + buf * C::UNIT;
+                uint16_t* Dr = Qr + C::RM_ELEMS;
+                uint16_t* Qt = Dr + C::RM_ELEMS;
+                uint16_t* Dt = Qt + C::TR_ELEMS;
+                const int cp = tid % C::NCP;
+#pragma unroll
+                for (int cb = 0; cb < C::COMBOS; ++cb) {
+                    const int rg = tid / C::NCP + cb * (NTHREADS / C::NCP);      // rows 4rg .. 4rg+3
+                    uint32_t qx[4], dx[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int r = 4 * rg + t;
+                        const int kr = r - delta + dc + BQ;                      // (i0 + r - delta) - kbase
+                        const uint32_t qa = *(const uint32_t*)(q_s + r * D + 2 * cp);
+                        const uint32_t ka = *(const uint32_t*)(k2_s + kr * D + 2 * cp);
+                        const uint32_t da = *(const uint32_t*)(do_s + r * D + 2 * cp);
+                        const uint32_t va = *(const uint32_t*)(v2_s + kr * D + 2 * cp);
+                        const float q0 = bf16_lo(qa) * (bf16_lo(ka) + p.k2_bias) * qscale;
+                        const float q1 = bf16_hi(qa) * (bf16_hi(ka) + p.k2_bias) * qscale;
+                        const float d0 = bf16_lo(da) * (bf16_lo(va) + p.v2_bias);
+                        const float d1 = bf16_hi(da) * (bf16_hi(va) + p.v2_bias);
+                        union { __bf16 h[2]; uint32_t u; } qq, dd;
+                        qq.h[0] = (__bf16)q0; qq.h[1] = (__bf16)q1;
+                        dd.h[0] = (__bf16)d0; dd.h[1] = (__bf16)d1;
+                        qx[t] = qq.u;
+                        dx[t] = dd.u;
+                        *(uint32_t*)(Qr + r * C::KS + 2 * cp) = qq.u;
+                        *(uint32_t*)(Dr + r * C::KS + 2 * cp) = dd.u;
+                    }
+                    // row r = 8g + 4hh + t sits at position (g/2)*16 + hh*8 + (g%2)*4 + t
+                    const int g = rg >> 1, hh = rg & 1;
+                    const int pos = (g >> 1) * 16 + hh * 8 + (g & 1) * 4;
+                    uint2 lo, hi;
+                    transpose4x2(qx, lo, hi);
+                    *(uint2*)(Qt + (2 * cp) * C::VS + pos) = lo;
+                    *(uint2*)(Qt + (2 * cp + 1) * C::VS + pos) = hi;
+                    transpose4x2(dx, lo, hi);
+                    *(uint2*)(Dt + (2 * cp) * C::VS + pos) = lo;
+                    *(uint2*)(Dt + (2 * cp + 1) * C::VS + pos) = hi;
+                }
+            };
+
+            form(dc, 0);
+            __syncthreads();
+            for (int x = 0; x < ndl; ++x) {
+                const int delta = dc + x;
+                if (x + 1 < ndl) form(delta + 1, (x + 1) & 1);
+                if (touches) {
+                    const uint16_t* Qr = units + (x & 1) * C::UNIT;
+                    const uint16_t* Dr = Qr + C::RM_ELEMS;
+                    const uint16_t* Qt = Dr + C::RM_ELEMS;
+                    const uint16_t* Dt = Qt + C::TR_ELEMS;
+                    // S[r, j] and dP[r, j]: rows = expanded rows, columns = this wavefront's K rows
+                    floatx16 sacc, dpacc;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) sacc[v] = dpacc[v] = 0.f;
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) {
+                        const bf16x8 qa = *(const bf16x8*)(Qr + ln * C::KS + kk * 16 + hf * 8);
+                        const bf16x8 da = *(const bf16x8*)(Dr + ln * C::KS + kk * 16 + hf * 8);
+                        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kfr[kk], sacc, 0, 0, 0);
+                        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vfr[kk], dpacc, 0, 0, 0);
+                    }
+                    float pv[16], dsv[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) pv[v] = sacc[v] - lse2r[v];
+                    const bool interior = (i0 >= jw + 31) && ((int64_t)i0 + 31 <= (int64_t)jw + w1) &&
+                                          (i0 + BQ - 1 < N) && (i0 >= delta);
+                    if (__builtin_expect(!interior, 0)) {
+                        // element v of this lane is query i0 + 8*(v/4) + 4*hf + v%4, column j
+                        const int lo = j - i0 - 4 * hf;            // need c >= lo
+                        const int hi = (int)((int64_t)j + w1 - i0 < 1 << 20 ? j + w1 - i0 : 1 << 20) - 4 * hf;
+                        const int dlo = delta - i0 - 4 * hf, nhi = N - 1 - i0 - 4 * hf;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = 8 * (v >> 2) + (v & 3);
+                            pv[v] = (j < N && c >= lo && c <= hi && c >= dlo && c <= nhi) ? pv[v] : -INFINITY;
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        pv[v] = fast_exp2(pv[v]);
+                        dsv[v] = pv[v] * (dpacc[v] - dsumr[v]);
+                    }
+                    bf16x8 pb[2], dsb[2];
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            pb[ks][t] = (__bf16)pv[ks * 8 + t];
+                            dsb[ks][t] = (__bf16)dsv[ks * 8 + t];
+                        }
+                    // dV^T[d, j] += dO~^T[d, r] P[r, j];  dK^T[d, j] += Q~^T[d, r] dS[r, j]
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks) {
+                            const bf16x8 dta = *(const bf16x8*)(Dt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                            const bf16x8 qta = *(const bf16x8*)(Qt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                            dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dta, pb[ks], dvacc[dt], 0, 0, 0);
+                            dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qta, dsb[ks], dkacc[dt], 0, 0, 0);
+                        }
+                }
+                __syncthreads();
+            }
+        }
+    }
+
+    if (j < N) {
+        uint16_t* dkp = p.dk1.p ? (uint16_t*)p.dk1.p + p.dk1.off(b, j, h) + 4 * hf : nullptr;
+        uint16_t* dvp = p.dv1.p ? (uint16_t*)p.dv1.p + p.dv1.off(b, j, h) + 4 * hf : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                union { __bf16 h[4]; uint2 u; } a, c;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    a.h[t] = (__bf16)(dkacc[dt][4 * g4 + t] * LN2);     // Q~ carries scale*log2(e)
+                    c.h[t] = (__bf16)dvacc[dt][4 * g4 + t];
+                }
+                if (dkp) *(uint2*)(dkp + dt * 32 + 8 * g4) = a.u;
+                if (dvp) *(uint2*)(dvp + dt * 32 + 8 * g4) = c.u;
+            }
+    }
+}
+
+template <int D>
+int launch_col_part(const Problem& p, hipStream_t st) {
+    using C = ColCfg<D>;
+    const int njb = (p.N + CJ - 1) / CJ;
+    const int64_t total = (int64_t)njb * p.B * p.H;
+    if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
+    if (hipFuncSetAttribute((const void*)mfma_bwd_col_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)C::LDS_BYTES) != hipSuccess)
+        return SA2_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL(mfma_bwd_col_kernel<D>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, njb,
+                       (int)total);
+    return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
+}
+
 size_t expanded_ws_bytes(int B, int N, int H, int D, int w2) {
     return (size_t)B * H * N * (size_t)(w2 + 1) * D * sizeof(uint16_t);
 }
@@ -366,10 +631,7 @@ int launch_mfma_bwd(const Problem& p, hipStream_t st) {
         if (rc != SA2_OK) return rc;
     }
     if (p.dk1.p || p.dv1.p) {
-        // column part: generic kernel until the MFMA column kernel lands
-        Problem g = p;
-        g.dq.p = g.dk2.p = g.dv2.p = nullptr;
-        rc = launch_generic_bwd(g, SA2_BF16, st);
+        rc = p.D == 128 ? launch_col_part<128>(p, st) : launch_col_part<64>(p, st);
     }
     return rc;
 }
