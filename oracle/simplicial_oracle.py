@@ -125,7 +125,12 @@ def forward_windowed(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias
         r = torch.matmul(w, v1f[:, :, None, j0:c1, :])                   # [B,H,i,k,D]
         num = (r * v2f[:, :, None, k0:c1, :]).sum(dim=3)                 # [B,H,i,D]
         outs.append(num / den[..., None])
-        lses.append(m[..., 0, 0] + torch.log(den))
+        # log(sum w + eps) for any m: when e^m underflows against eps, factor eps out instead
+        mm, l = m[..., 0, 0], w.sum(dim=(-1, -2))
+        log_eps = math.log(eps)
+        hi = mm + torch.log(l + eps * torch.exp(-mm.clamp_min(log_eps)))
+        lo = log_eps + torch.log1p(l * torch.exp(mm.clamp_max(log_eps) - log_eps))
+        lses.append(torch.where(mm > log_eps, hi, lo))
     out = torch.cat(outs, dim=2).permute(0, 2, 1, 3)                     # [B,n,H,D]
     lse = torch.cat(lses, dim=2)                                         # [B,H,n]
     return out, lse

@@ -55,8 +55,11 @@ def test_window_sizes(w):
     inp = make_inputs(2, 96, 2, 32, seed=7)
     got = run_device(inp, w[0], w[1], flags=GENERIC)
     want = oracle_all(inp, w[0], w[1])
+    # single-triple windows: dq, dk, dk' vanish by cancellation (only the 1e-8 epsilon
+    # keeps them from being exactly 0); what the fp32 kernels return is rounding noise
+    atol = 1e-5 if w == (0, 0) else 1e-6
     for name in ("out", "lse", "dq", "dk1", "dk2", "dv1", "dv2"):
-        assert_close_rel(got[name], want[name], 2e-5, name)
+        assert_close_rel(got[name], want[name], 2e-5, name, atol=atol)
 
 
 @pytest.mark.parametrize("bias", [(0.0, 0.0), (0.1, 0.2), (-0.1, -0.2), (1.0, 0.5)])

@@ -141,7 +141,7 @@ def test_row_zero_and_epsilon():
     negative logit the epsilon dominates and the output collapses to 0."""
     B, N, H, D = 1, 4, 1, 4
     q, k1, k2, v1, v2 = five(B, N, H, D, seed=9)
-    for scale in (0.5, -40.0, -400.0):
+    for scale in (0.5, -40.0, -400.0, -40000.0):
         s = (q[:, 0] * k1[:, 0] * k2[:, 0]).sum(-1, keepdim=True).abs() * scale
         q0 = q.clone()
         q0[:, 0] = q[:, 0] * torch.sign((q[:, 0] * k1[:, 0] * k2[:, 0]).sum(-1, keepdim=True))
