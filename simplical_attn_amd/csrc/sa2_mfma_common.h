@@ -8,11 +8,13 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 constexpr int BQ = 32;       // queries per workgroup
 constexpr int TJ = 32;       // keys per LDS tile
 constexpr int NTHREADS = 256;
 constexpr float RESCALE_LOG2 = 8.0f;
+constexpr float OVERFLOW_LIMIT = 1.0e30f;    // a row sum above this means a stale softmax reference point
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 constexpr float LOG2_EPS = -26.575424759098897f;   // log2(1e-8)

@@ -4,26 +4,33 @@
 // delta = i - k in [0, w2], with Q~[r,:] = q[i,:] * (k2[i-delta,:] + k2_bias) *
 // scale*log2(e), rounded to bf16.  Then s[r,j] = Q~[r].k1[j] and
 // R[r,:] = sum_j p[r,j] v1[j,:] are sliding-window flash attention on the
-// expanded rows (both contractions on v_mfma_f32_32x32x16_bf16, fp32 online
-// softmax per row), and the rows of a query are merged at the end with a
-// second online softmax:  O[i] = sum_delta e^{m_r-M} (v2[i-delta]+v2_bias) * R[r]
-// / (L + 1e-8 e^{-M}).  No logit outside the K' window is ever computed.
+// expanded rows (both contractions on v_mfma_f32_32x32x16_bf16, fp32 softmax
+// per row), and the rows of a query are merged with a second online softmax:
+// O[i] = sum_delta e^{m_r-M} (v2[i-delta]+v2_bias) * R[r] / (L + 1e-8 e^{-M}).
+// No logit outside the K' window is ever computed.
 //
-// Work split: one workgroup (4 wavefronts) owns 32 consecutive queries of one
-// (batch, head).  A "unit" is (delta, those 32 queries) = one 32-row MFMA
-// N-tile.  A wavefront holds two units at a time (they share every K/V operand
-// fetched from LDS) and sweeps the K window [i0-w1, i0+31] in 32-key tiles that
-// the workgroup stages through double-buffered LDS: K row-major, V transposed
-// and permuted so that each MFMA operand is one 16-byte LDS read.
+// Work split: one workgroup of 8 wavefronts (two per SIMD, so that one
+// wavefront's softmax arithmetic overlaps the other's MFMAs) owns 32 consecutive
+// queries of one (batch, head).  A "unit" is (delta, those 32 queries) = one
+// 32-row MFMA N-tile; each wavefront holds one unit at a time and sweeps the K
+// window [i0-w1, i0+31] in 32-key tiles that the workgroup stages through
+// double-buffered LDS: K row-major, V transposed and permuted so that every
+// MFMA operand is one 16-byte LDS read.  After each round of 8 units the
+// wavefronts fold their (m, l, R*v2) into the workgroup's fp32 accumulator
+// through bf16 slabs in LDS, each thread summing a fixed slice in a fixed order.
 //
 // The logits are computed transposed (S^T = K1 . Q~^T) so that an expanded row
-// lives in one lane (pair): row maxima and sums are in-lane reductions plus one
-// exchange with lane^32, and exp2(S^T) is already laid out as the B operand of
-// R^T = V^T . P^T.
+// lives in one lane pair: exp2(S^T) is already laid out as the B operand of
+// R^T = V^T . P^T.  The softmax reference point of a unit is fixed at the first
+// tile that holds one of its keys and enters the logit MFMA as its C operand, so
+// on unmasked tiles the vector ALU only does exp2, bf16 packing and a row sum.
 #include "sa2_mfma_common.h"
 
 namespace sa2 {
 namespace {
+
+constexpr int FW = 8;                 // wavefronts per workgroup
+constexpr int FT = FW * 64;           // threads per workgroup
 
 template <int D>
 struct Cfg {
@@ -34,21 +41,37 @@ struct Cfg {
     static constexpr int K_ELEMS = TJ * KS;
     static constexpr int V_ELEMS = D * VS;
     static constexpr int STAGE = K_ELEMS + V_ELEMS;
-    static constexpr int KR = TJ * D / 8 / NTHREADS;       // 16-byte K chunks per thread per tile
+    static constexpr int KCH = TJ * D / 8;                  // 16-byte K chunks per tile
     static constexpr int NDP = D / 2;                       // column pairs of V
-    static constexpr int VPASS = NDP / 32;                  // 4-row groups per thread per tile
-    static constexpr int OS = D + 4;                        // merge buffer row stride (fp32)
-    static constexpr int MERGE_FLOATS = 4 * (BQ * OS + 2 * BQ);
-    static constexpr size_t STAGE_BYTES = (size_t)2 * STAGE * 2;          // two staging buffers
-    static constexpr size_t LDS_BYTES = STAGE_BYTES + (size_t)MERGE_FLOATS * 4;
+    static constexpr int SS = D + 8;                        // slab row stride (bf16)
+    static constexpr int OS = D + 4;                        // accumulator row stride (fp32)
+    // LDS carve-up (bytes)
+    static constexpr size_t STAGE_BYTES = (size_t)2 * STAGE * 2;
+    static constexpr size_t SLAB_BYTES = (size_t)FW * BQ * SS * 2;
+    static constexpr size_t OACC_BYTES = (size_t)BQ * OS * 4;
+    static constexpr size_t XCH_BYTES = (size_t)(2 * FW * BQ + 3 * BQ) * 4;
+    static constexpr size_t LDS_BYTES = STAGE_BYTES + SLAB_BYTES + OACC_BYTES + XCH_BYTES;
 };
 
-template <int D>
-__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+// SAFE = false: the fast kernel.  A weight that overflows (logits growing by more
+// than ~100 octaves along the window after the reference point was fixed) only marks
+// the block by storing NaN in its first LSE slot.
+// SAFE = true: the repair kernel, launched right after: a block that finds the mark
+// recomputes itself refreshing the reference point on every tile; every other block
+// exits at once.
+template <int D, bool SAFE>
+__global__ __launch_bounds__(FT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void mfma_fwd_kernel(Problem p, int nqb, int total) {
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* smem = (uint16_t*)smem_raw;
+    uint16_t* slabs = (uint16_t*)(smem_raw + C::STAGE_BYTES);
+    float* oacc = (float*)(smem_raw + C::STAGE_BYTES + C::SLAB_BYTES);
+    float* xch_m = oacc + BQ * C::OS;           // [FW][BQ]
+    float* xch_l = xch_m + FW * BQ;             // [FW][BQ]
+    float* xch_a = xch_l + FW * BQ;             // [BQ] accumulator rescale of this round
+    float* fin_m = xch_a + BQ;                  // [BQ] final M
+    float* fin_l = fin_m + BQ;                  // [BQ] final L
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -66,6 +89,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     const int i = i0 + ln;
     const int ic = i < N ? i : N - 1;
     const int i_last = (i0 + BQ - 1 < N ? i0 + BQ - 1 : N - 1);
+    if (SAFE) {
+        const float mark = p.lse[(int64_t)bh * N + i0];
+        if (mark == mark) return;                 // not NaN: the fast kernel's result stands
+    }
 
     const uint16_t* qp = (const uint16_t*)p.q.p + p.q.off(b, 0, h);
     const uint16_t* k1p = (const uint16_t*)p.k1.p + p.k1.off(b, 0, h);
@@ -77,75 +104,73 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     const int jt_hi = i_last / TJ;
     const int nt = jt_hi - jt_lo + 1;
     const int n_units = (w2 < i_last ? w2 : i_last) + 1;     // delta = 0 .. n_units-1
-    const int npairs = (n_units + 1) >> 1;
-    const int nrounds = (npairs + 3) >> 2;
+    const int nrounds = (n_units + FW - 1) / FW;
     const int total_steps = nrounds * nt;
 
     // ---- staging of one K/V tile: global -> registers -> LDS ----------------
-    uint4 kreg[C::KR];
-    uint32_t vreg[C::VPASS * 4];
-    const int v_dp = tid % C::NDP, v_g0 = tid / C::NDP;
+    // K: KCH 16-byte chunks, V: 8 four-row groups x NDP column pairs; one of each
+    // per thread when D = 128, the first half of the threads when D = 64.
+    const bool k_owner = tid < C::KCH;
+    const int k_row = tid / (D / 8), k_col = tid - k_row * (D / 8);
+    const bool v_owner = tid < 8 * C::NDP;
+    const int v_dp = tid % C::NDP, v_grp = tid / C::NDP;
+    const uint32_t k_off = (uint32_t)k_row * (uint32_t)p.k1.sn + k_col * 8;
+    const uint32_t v_off = (uint32_t)(v_grp * 4) * (uint32_t)p.v1.sn + 2 * v_dp;
+    const uint32_t v_sn = (uint32_t)p.v1.sn;
+    uint4 kreg = make_uint4(0u, 0u, 0u, 0u);
+    uint32_t vreg[4] = {0u, 0u, 0u, 0u};
     auto load_tile = [&](int jt) {
         const int j0 = jt * TJ;
+        if (__builtin_expect(j0 + TJ <= N, 1)) {
+            if (k_owner) kreg = *(const uint4*)(k1p + (int64_t)j0 * p.k1.sn + k_off);
+            if (v_owner) {
+                const uint16_t* vb = v1p + (int64_t)j0 * p.v1.sn + v_off;
 #pragma unroll
-        for (int u = 0; u < C::KR; ++u) {
-            const int c = tid + NTHREADS * u;
-            const int row = c / (D / 8), col = c - row * (D / 8);
-            int j = j0 + row;
-            j = j < N ? j : N - 1;
-            kreg[u] = *(const uint4*)(k1p + (int64_t)j * p.k1.sn + col * 8);
-        }
-#pragma unroll
-        for (int ps = 0; ps < C::VPASS; ++ps) {
-            const int grp = v_g0 + ps * (NTHREADS / C::NDP);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                int j = j0 + grp * 4 + r;
+                for (int r = 0; r < 4; ++r) vreg[r] = *(const uint32_t*)(vb + r * v_sn);
+            }
+        } else {
+            // last tile of the sequence: clamp the rows (they are masked later)
+            if (k_owner) {
+                int j = j0 + k_row;
                 j = j < N ? j : N - 1;
-                vreg[ps * 4 + r] = *(const uint32_t*)(v1p + (int64_t)j * p.v1.sn + 2 * v_dp);
+                kreg = *(const uint4*)(k1p + (int64_t)j * p.k1.sn + k_col * 8);
+            }
+            if (v_owner) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int j = j0 + v_grp * 4 + r;
+                    j = j < N ? j : N - 1;
+                    vreg[r] = *(const uint32_t*)(v1p + (int64_t)j * p.v1.sn + 2 * v_dp);
+                }
             }
         }
     };
     auto store_tile = [&](int buf) {
         uint16_t* Ks = smem + buf * C::STAGE;
         uint16_t* Vt = Ks + C::K_ELEMS;
-#pragma unroll
-        for (int u = 0; u < C::KR; ++u) {
-            const int c = tid + NTHREADS * u;
-            const int row = c / (D / 8), col = c - row * (D / 8);
-            *(uint4*)(Ks + row * C::KS + col * 8) = kreg[u];
-        }
-#pragma unroll
-        for (int ps = 0; ps < C::VPASS; ++ps) {
-            const int grp = v_g0 + ps * (NTHREADS / C::NDP);
+        if (k_owner) *(uint4*)(Ks + k_row * C::KS + k_col * 8) = kreg;
+        if (v_owner) {
             // key j = 8g + 4hh + t of the tile sits at position (g/2)*16 + hh*8 + (g%2)*4 + t
-            const int g = grp >> 1, hh = grp & 1;
+            const int g = v_grp >> 1, hh = v_grp & 1;
             const int pos = (g >> 1) * 16 + hh * 8 + (g & 1) * 4;
-            const uint32_t x0 = vreg[ps * 4], x1 = vreg[ps * 4 + 1], x2 = vreg[ps * 4 + 2], x3 = vreg[ps * 4 + 3];
             uint2 lo, hi;
-            lo.x = (x0 & 0xffffu) | (x1 << 16);
-            lo.y = (x2 & 0xffffu) | (x3 << 16);
-            hi.x = (x0 >> 16) | (x1 & 0xffff0000u);
-            hi.y = (x2 >> 16) | (x3 & 0xffff0000u);
+            lo.x = (vreg[0] & 0xffffu) | (vreg[1] << 16);
+            lo.y = (vreg[2] & 0xffffu) | (vreg[3] << 16);
+            hi.x = (vreg[0] >> 16) | (vreg[1] & 0xffff0000u);
+            hi.y = (vreg[2] >> 16) | (vreg[3] & 0xffff0000u);
             *(uint2*)(Vt + (2 * v_dp) * C::VS + pos) = lo;
             *(uint2*)(Vt + (2 * v_dp + 1) * C::VS + pos) = hi;
         }
     };
 
-    // ---- per-wavefront state -------------------------------------------------
-    // The query accumulators O (fp32, unnormalised, relative to Mrun) live in
-    // LDS behind the staging buffers: they are touched once per unit, and the
-    // registers they would take are what keeps the sweep free of AGPR copies.
-    float* fm = (float*)(smem_raw + C::STAGE_BYTES);
-    float* Om = fm + wave * (BQ * C::OS + 2 * BQ);
-    float* Mm = Om + BQ * C::OS;
-    float* Lm = Mm + BQ;
+    // ---- workgroup accumulators ------------------------------------------------
+    // thread -> (query aq, ACN columns from ac) of the fp32 accumulator in LDS
+    constexpr int ACN = D / 16;                    // columns per thread (8 or 4)
+    const int aq = tid >> 4, ac = (tid & 15) * ACN;
 #pragma unroll
-    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4)
-            *(float4*)(Om + ln * C::OS + dt * 32 + 8 * g4 + 4 * hf) = make_float4(0.f, 0.f, 0.f, 0.f);
-    float Mrun = -INFINITY, Lrun = 0.f;
+    for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = 0.f;
+    float Mrun = -INFINITY, Lrun = 0.f;            // per query (lane), replicated in every wavefront
+    bool bad = false;
 
     const float qscale = p.scale * LOG2E;
 
@@ -154,227 +179,285 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     if (total_steps > 1) load_tile(jt_lo + (1 % nt));
     __syncthreads();
 
+    // Tiles [s_lo, s_hi] need no mask: every key of the tile is inside the K window of
+    // every query of the block.
+    int s_lo = (i0 + BQ - 1 - w1 + TJ - 1) / TJ - jt_lo;       // first tile with j0 >= i0+31-w1
+    s_lo = (i0 + BQ - 1 - w1 <= jt_lo * TJ) ? 0 : s_lo;
+    const int s_hi = (i0 + 1) / TJ - 1 - jt_lo;                 // last tile with j0+31 <= i0
+
     int g = 0;
     for (int round = 0; round < nrounds; ++round) {
-        const int pair = round * 4 + wave;
-        const int delta0 = 2 * pair, delta1 = 2 * pair + 1;
-        const bool ok0 = delta0 < n_units, ok1 = delta1 < n_units;
+        const int delta = round * FW + wave;
+        const bool ok = delta < n_units;
+        float m = -INFINITY, l = 0.f;
+        floatx16 racc[C::DT];
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) racc[dt][v] = 0.f;
 
-        if (!ok0) {
-            // nothing to compute this round: keep the staging pipeline moving
+        if (!ok) {
+            // no unit for this wavefront in this round: keep the staging pipeline moving
             for (int s = 0; s < nt; ++s, ++g) {
                 if (g + 1 < total_steps) store_tile((g + 1) & 1);
                 if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
                 __syncthreads();
             }
-            continue;
-        }
-
-        // ---- new pair of units: Q~ operands, fresh running softmax ----------
-        bf16x8 qf[2][C::DK];
-        floatx16 racc[2][C::DT];
-        float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+        } else {
+            // ---- new unit: Q~ operand, fresh softmax state ----------------------
+            bf16x8 qf[C::DK];
+            {
+                int k = ic - delta;
+                k = k > 0 ? k : 0;
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+                for (int kk = 0; kk < C::DK; ++kk) {
+                    const uint4 qa = *(const uint4*)(qp + (int64_t)ic * p.q.sn + kk * 16 + hf * 8);
+                    const uint4 kb = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + kk * 16 + hf * 8);
+                    const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
+                    const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
+                    bf16x8 r;
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) racc[u][dt][v] = 0.f;
-            int k = ic - (u ? delta1 : delta0);
-            k = k > 0 ? k : 0;
-#pragma unroll
-            for (int kk = 0; kk < C::DK; ++kk) {
-                const uint4 qa = *(const uint4*)(qp + (int64_t)ic * p.q.sn + kk * 16 + hf * 8);
-                const uint4 kb = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + kk * 16 + hf * 8);
-                const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
-                const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
-                bf16x8 r;
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
-                    r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
-                }
-                qf[u][kk] = r;
-            }
-        }
-        const bool rows_full0 = i0 >= delta0 && i0 + BQ - 1 < N;
-        const bool rows_full1 = ok1 && i0 >= delta1 && i0 + BQ - 1 < N;
-        const bool row_ok0 = i < N && i >= delta0;
-        const bool row_ok1 = ok1 && i < N && i >= delta1;
-
-        for (int s = 0; s < nt; ++s, ++g) {
-            const int j0 = (jt_lo + s) * TJ;
-            const uint16_t* Ks = smem + (g & 1) * C::STAGE;
-            const uint16_t* Vt = Ks + C::K_ELEMS;
-            // S^T tiles: rows = keys of the tile, columns = expanded rows
-            floatx16 sacc[2];
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) sacc[u][v] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < C::DK; ++kk) {
-                const bf16x8 ka = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
-                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[0][kk], sacc[0], 0, 0, 0);
-                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[1][kk], sacc[1], 0, 0, 0);
-            }
-            const bool interior = (j0 + TJ - 1 <= i0) && (j0 >= i0 + BQ - 1 - w1);
-            bf16x8 pb[2][2];
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                float pv[16];
-#pragma unroll
-                for (int v = 0; v < 16; ++v) pv[v] = sacc[u][v];
-                if (__builtin_expect(!(interior && (u ? rows_full1 : rows_full0)), 0)) {
-                    // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
-                    const bool row_ok = u ? row_ok1 : row_ok0;
-                    const int hi = i - j0 - 4 * hf, lo = hi - w1;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int c = 8 * (v >> 2) + (v & 3);
-                        pv[v] = (row_ok && c <= hi && c >= lo) ? pv[v] : -INFINITY;
+                    for (int t = 0; t < 4; ++t) {
+                        r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
+                        r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
                     }
+                    qf[kk] = r;
                 }
-                float mx = fmaxf(pv[0], pv[1]);
+            }
+            const bool rows_full = i0 >= delta && i0 + BQ - 1 < N;
+            const bool row_ok = i < N && i >= delta;
+            // -m (0 while the row has no finite logit yet), as a scalar and replicated over an
+            // accumulator tuple: the tuple is the C operand of the first logit MFMA.
+            float nm = 0.f;
+            floatx16 negm;
 #pragma unroll
-                for (int v = 2; v < 16; ++v) mx = fmaxf(mx, pv[v]);
-                mx = fmaxf(mx, other_half(mx));
-                // Lazy reference point: move it only when the maximum grows by more
-                // than 2^RESCALE_LOG2, so the accumulator rescale is rare; weights
-                // stay below 2^RESCALE_LOG2 and every later formula only needs m to
-                // be a common reference, not the exact maximum.
-                if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[u] + RESCALE_LOG2) != 0, 0)) {
-                    const float m_new = (mx > m[u] + RESCALE_LOG2) ? mx : m[u];
-                    const float alpha = fast_exp2(m[u] - ((m_new == -INFINITY) ? 0.f : m_new));
-                    m[u] = m_new;
-                    l[u] *= alpha;
-                    asm volatile("s_nop 15\n\ts_nop 15");
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt) scale_acc(racc[u][dt], alpha);
-                    asm volatile("s_nop 4");
-                }
-                const float m_use = (m[u] == -INFINITY) ? 0.f : m[u];
-                float rs = 0.f;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    pv[v] = fast_exp2(pv[v] - m_use);
-                    rs += pv[v];
-                }
-                l[u] += rs;
+            for (int v = 0; v < 16; ++v) negm[v] = 0.f;
+
+            // exp2 of the shifted logits -> bf16 weights (MFMA B operand) and their row sum
+            auto weights = [&](const floatx16& sh, bf16x8* w, float& rsum) {
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) pb[u][ks][t] = (__bf16)pv[ks * 8 + t];
+                    for (int t = 0; t < 8; ++t) w[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t]);
+                const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
+                float r = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 0, 1), ones, r, false);
+                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 2, 3), ones, r, false);
+                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 4, 5), ones, r, false);
+                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 6, 7), ones, r, false);
+                }
+                rsum = r;
+            };
+            auto value_mfmas = [&](const uint16_t* Vt, const bf16x8* w) {
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const bf16x8 va = *(const bf16x8*)(Vt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                        racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, w[ks], racc[dt], 0, 0, 0);
+                    }
+            };
+
+            const int fast_lo = (!SAFE && rows_full) ? (s_lo > 1 ? s_lo : 1) : nt;
+            const int fast_hi = (!SAFE && rows_full) ? s_hi + 1 : nt;   // exclusive
+
+            int s = 0;
+            while (s < nt) {
+                if (s < fast_lo || s >= fast_hi) {
+                    // ---- general tile: masks, and a (new) reference point where needed ----
+                    const int j0 = (jt_lo + s) * TJ;
+                    const uint16_t* Ks = smem + (g & 1) * C::STAGE;
+                    const uint16_t* Vt = Ks + C::K_ELEMS;
+                    const bool plain = (j0 + TJ - 1 <= i0) && (j0 >= i0 + BQ - 1 - w1) && rows_full;
+                    // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
+                    const int hi = i - j0 - 4 * hf, lo = hi - w1;
+                    bf16x8 ka[C::DK];
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+                    if (SAFE || s == 0 || __builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
+                        floatx16 t;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) t[v] = 0.f;
+#pragma unroll
+                        for (int kk = 0; kk < C::DK; ++kk)
+                            t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], t, 0, 0, 0);
+                        float mx = -INFINITY;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = 8 * (v >> 2) + (v & 3);
+                            const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
+                            mx = fmaxf(mx, valid ? t[v] : -INFINITY);
+                        }
+                        mx = fmaxf(mx, other_half(mx));
+                        // Lazy: move the reference only when the maximum grew by more than
+                        // 2^RESCALE_LOG2; later formulas only need m as a common reference.
+                        const float m_new = (mx > m + RESCALE_LOG2) ? mx : m;
+                        if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+                            const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
+                            m = m_new;
+                            l *= alpha;
+                            if (s > 0) {
+#pragma unroll
+                                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                                    for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
+                            }
+                            nm = (m_new == -INFINITY) ? 0.f : -m_new;
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) negm[v] = nm;
+                        }
+                    }
+                    floatx16 ct;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int c = 8 * (v >> 2) + (v & 3);
+                        const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
+                        ct[v] = valid ? nm : -INFINITY;
+                    }
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk)
+                        ct = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], ct, 0, 0, 0);
+                    bf16x8 pb[2];
+                    float rs;
+                    weights(ct, pb, rs);
+                    l += rs;
+                    bad |= !(rs < OVERFLOW_LIMIT);
+                    value_mfmas(Vt, pb);
+                    if (g + 1 < total_steps) store_tile((g + 1) & 1);
+                    if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
+                    __syncthreads();
+                    ++s;
+                    ++g;
+                    continue;
+                }
+                // ---- unmasked tiles: reference point fixed, straight-line body ----
+                for (; s < fast_hi; ++s, ++g) {
+                    const uint16_t* Ks = smem + (g & 1) * C::STAGE;
+                    const uint16_t* Vt = Ks + C::K_ELEMS;
+                    floatx16 sh = negm;
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) {
+                        const bf16x8 ka = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], sh, 0, 0, 0);
+                    }
+                    bf16x8 pb[2];
+                    float rs;
+                    weights(sh, pb, rs);
+                    l += rs;
+                    bad |= !(rs < OVERFLOW_LIMIT);
+                    value_mfmas(Vt, pb);
+                    if (g + 1 < total_steps) store_tile((g + 1) & 1);
+                    if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
+                    __syncthreads();
+                }
             }
-            // R^T += V^T . P^T
+        }
+
+        // ---- fold the round's units into the workgroup accumulator --------------
+        const float lt = l + other_half(l);
+        if (hf == 0) {
+            xch_m[wave * BQ + ln] = m;
+            xch_l[wave * BQ + ln] = lt;
+        }
+        __syncthreads();
+        float Mn = Mrun;
+#pragma unroll
+        for (int w = 0; w < FW; ++w) Mn = fmaxf(Mn, xch_m[w * BQ + ln]);
+        const float Muse = (Mn == -INFINITY) ? 0.f : Mn;
+        const float a = fast_exp2(Mrun - Muse);
+        float Ln = Lrun * a;
+#pragma unroll
+        for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln] * fast_exp2(xch_m[w * BQ + ln] - Muse);
+        Mrun = Mn;
+        Lrun = Ln;
+        if (wave == 0 && hf == 0) xch_a[ln] = a;
+        {
+            // this wavefront's contribution, bf16, to its slab: c * (v2 + bias) * R
+            const float cw = ok ? fast_exp2(m - Muse) : 0.f;
+            int kr = ic - delta;
+            kr = kr > 0 ? kr : 0;
+            const uint16_t* vrow = v2p + (int64_t)kr * p.v2.sn + 4 * hf;
+            uint16_t* srow = slabs + (wave * BQ + ln) * C::SS + 4 * hf;
 #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const bf16x8 va = *(const bf16x8*)(Vt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
-                    racc[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][ks], racc[0][dt], 0, 0, 0);
-                    racc[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][ks], racc[1][dt], 0, 0, 0);
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    uint2 x = make_uint2(0u, 0u);
+                    if (ok) x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                    union { __bf16 h[4]; uint2 u; } o;
+                    o.h[0] = (__bf16)(cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
+                    o.h[1] = (__bf16)(cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
+                    o.h[2] = (__bf16)(cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
+                    o.h[3] = (__bf16)(cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
+                    *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
                 }
-
-            if (g + 1 < total_steps) store_tile((g + 1) & 1);
-            if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
-            __syncthreads();
         }
-
-        // ---- fold the finished units into the query accumulators ------------
-        float a_all = 1.f, bb[2];
+        __syncthreads();
+        {
+            // each thread sums its slice of the 8 slabs in wavefront order
+            const float ar = xch_a[aq];
+            float acc[ACN];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const float lt = l[u] + other_half(l[u]);
-            const float Mn = fmaxf(Mrun, m[u]);
-            const float Muse = (Mn == -INFINITY) ? 0.f : Mn;
-            const float a = fast_exp2(Mrun - Muse);
-            bb[u] = fast_exp2(m[u] - Muse);
-            // unit 0's factor must also shrink by unit 1's rescale of the accumulator
-            if (u == 1) bb[0] *= a;
-            a_all *= a;
-            Lrun = Lrun * a + lt * bb[u];
-            Mrun = Mn;
-        }
-        int kr0 = ic - delta0, kr1 = ic - delta1;
-        kr0 = kr0 > 0 ? kr0 : 0;
-        kr1 = kr1 > 0 ? kr1 : 0;
-        const uint16_t* vrow0 = v2p + (int64_t)kr0 * p.v2.sn + 4 * hf;
-        const uint16_t* vrow1 = v2p + (int64_t)kr1 * p.v2.sn + 4 * hf;
+            for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c] * ar;
 #pragma unroll
-        for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const uint2 x0 = *(const uint2*)(vrow0 + dt * 32 + 8 * g4);
-                const uint2 x1 = *(const uint2*)(vrow1 + dt * 32 + 8 * g4);
-                float* op = Om + ln * C::OS + dt * 32 + 8 * g4 + 4 * hf;
-                float4 o = *(float4*)op;
-                const float b0 = bb[0], b1 = bb[1];
-                o.x = o.x * a_all + b0 * racc[0][dt][4 * g4 + 0] * (bf16_lo(x0.x) + p.v2_bias) +
-                      b1 * racc[1][dt][4 * g4 + 0] * (bf16_lo(x1.x) + p.v2_bias);
-                o.y = o.y * a_all + b0 * racc[0][dt][4 * g4 + 1] * (bf16_hi(x0.x) + p.v2_bias) +
-                      b1 * racc[1][dt][4 * g4 + 1] * (bf16_hi(x1.x) + p.v2_bias);
-                o.z = o.z * a_all + b0 * racc[0][dt][4 * g4 + 2] * (bf16_lo(x0.y) + p.v2_bias) +
-                      b1 * racc[1][dt][4 * g4 + 2] * (bf16_lo(x1.y) + p.v2_bias);
-                o.w = o.w * a_all + b0 * racc[0][dt][4 * g4 + 3] * (bf16_hi(x0.y) + p.v2_bias) +
-                      b1 * racc[1][dt][4 * g4 + 3] * (bf16_hi(x1.y) + p.v2_bias);
-                *(float4*)op = o;
+            for (int w = 0; w < FW; ++w) {
+                const uint16_t* sp = slabs + (w * BQ + aq) * C::SS + ac;
+                if (ACN == 8) {
+                    const uint4 x = *(const uint4*)sp;
+                    acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
+                    acc[4 % ACN] += bf16_lo(x.z); acc[5 % ACN] += bf16_hi(x.z);
+                    acc[6 % ACN] += bf16_lo(x.w); acc[7 % ACN] += bf16_hi(x.w);
+                } else {
+                    const uint2 x = *(const uint2*)sp;
+                    acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
+                }
             }
+#pragma unroll
+            for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
+        }
+        // (the slabs and exchange arrays are next written a whole tile sweep of barriers later)
     }
 
-    // ---- merge the four wavefronts' partial (M, L, O) through LDS ------------
-    if (hf == 0) {
-        Mm[ln] = Mrun;
-        Lm[ln] = Lrun;
+    // ---- normalise and store ------------------------------------------------------
+    const bool any_bad = !SAFE && __syncthreads_or(bad ? 1 : 0);
+    if (wave == 0 && hf == 0) {
+        fin_m[ln] = Mrun;
+        fin_l[ln] = Lrun;
     }
     __syncthreads();
-
-    constexpr int CH = D / 8;                 // output columns per thread
-    const int qi = tid >> 3, dc = (tid & 7) * CH;
-    const int io = i0 + qi;
+    const int io = i0 + aq;
     if (io < N) {
-        float Mw[4], Ms = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            Mw[w] = fm[w * (BQ * C::OS + 2 * BQ) + BQ * C::OS + qi];
-            Ms = fmaxf(Ms, Mw[w]);
-        }
-        float cw[4], L = 0.f;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            cw[w] = fast_exp2(Mw[w] - Ms);    // a wavefront without units has M = -inf -> weight 0
-            L += cw[w] * fm[w * (BQ * C::OS + 2 * BQ) + BQ * C::OS + BQ + qi];
-        }
+        const float Ms = fin_m[aq], L = fin_l[aq];
         const float inv = 1.f / (L + 1e-8f * fast_exp2(-Ms));
-        uint16_t* orow = (uint16_t*)p.out.p + p.out.off(b, io, h) + dc;
+        uint16_t* orow = (uint16_t*)p.out.p + p.out.off(b, io, h) + ac;
+        union { __bf16 h[8]; uint4 u4; uint2 u2; } o;
 #pragma unroll
-        for (int c4 = 0; c4 < CH; c4 += 8) {
-            bf16x8 r;
-#pragma unroll
-            for (int t4 = 0; t4 < 8; t4 += 4) {
-                float4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const float4 x = *(const float4*)(fm + w * (BQ * C::OS + 2 * BQ) + qi * C::OS + dc + c4 + t4);
-                    acc.x += cw[w] * x.x;
-                    acc.y += cw[w] * x.y;
-                    acc.z += cw[w] * x.z;
-                    acc.w += cw[w] * x.w;
-                }
-                r[t4 + 0] = (__bf16)(acc.x * inv);
-                r[t4 + 1] = (__bf16)(acc.y * inv);
-                r[t4 + 2] = (__bf16)(acc.z * inv);
-                r[t4 + 3] = (__bf16)(acc.w * inv);
-            }
-            *(bf16x8*)(orow + c4) = r;
-        }
-        if ((tid & 7) == 0) {
+        for (int c = 0; c < ACN; ++c) o.h[c] = (__bf16)(oacc[aq * C::OS + ac + c] * inv);
+        if (ACN == 8) *(uint4*)orow = o.u4;
+        else *(uint2*)orow = o.u2;
+        if ((tid & 15) == 0) {
             float lse;
             if (Ms > LOG2_EPS) lse = LN2 * (Ms + __log2f(L + 1e-8f * fast_exp2(-Ms)));
             else lse = LN_EPS + log1pf(L * fast_exp2(Ms - LOG2_EPS));
-            p.lse[(int64_t)bh * N + io] = lse;
+            p.lse[(int64_t)bh * N + io] = (any_bad && aq == 0) ? __builtin_nanf("") : lse;
         }
     }
+}
+
+template <int D>
+int launch_fwd_pair(const Problem& p, int nqb, int total, hipStream_t st) {
+    using C = Cfg<D>;
+    if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)C::LDS_BYTES) != hipSuccess ||
+        hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)C::LDS_BYTES) != hipSuccess)
+        return SA2_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL((mfma_fwd_kernel<D, false>), dim3((unsigned)total), dim3(FT), C::LDS_BYTES, st, p, nqb, total);
+    if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL((mfma_fwd_kernel<D, true>), dim3((unsigned)total), dim3(FT), C::LDS_BYTES, st, p, nqb, total);
+    return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
 
 bool aligned16(const Tensor& t, int B, int N, int H) {
@@ -383,6 +466,8 @@ bool aligned16(const Tensor& t, int B, int N, int H) {
     if (B > 1 && (t.sb & 7)) return false;
     if (N > 1 && (t.sn & 7)) return false;
     if (H > 1 && (t.sh & 7)) return false;
+    // the kernels address rows of one (batch, head) slice with 32-bit element offsets
+    if (N > 1 && (int64_t)(N - 1) * t.sn + 256 >= (int64_t)1 << 31) return false;
     return true;
 }
 
@@ -409,22 +494,7 @@ int launch_mfma_fwd(const Problem& p, hipStream_t st) {
     const int nqb = (p.N + BQ - 1) / BQ;
     const int64_t total = (int64_t)nqb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-    if (p.D == 128) {
-        using C = Cfg<128>;
-        if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)C::LDS_BYTES) != hipSuccess)
-            return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL(mfma_fwd_kernel<128>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, nqb,
-                           (int)total);
-    } else {
-        using C = Cfg<64>;
-        if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)C::LDS_BYTES) != hipSuccess)
-            return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL(mfma_fwd_kernel<64>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, nqb,
-                           (int)total);
-    }
-    return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
+    return p.D == 128 ? launch_fwd_pair<128>(p, nqb, (int)total, st) : launch_fwd_pair<64>(p, nqb, (int)total, st);
 }
 
 }  // namespace sa2
