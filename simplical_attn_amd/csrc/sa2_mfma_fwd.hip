@@ -13,11 +13,15 @@
 // wavefront's softmax arithmetic overlaps the other's MFMAs) owns 32 consecutive
 // queries of one (batch, head).  A "unit" is (delta, those 32 queries) = one
 // 32-row MFMA N-tile; each wavefront holds one unit at a time and sweeps the K
-// window [i0-w1, i0+31] in 32-key tiles that the workgroup stages through
-// double-buffered LDS: K row-major, V transposed and permuted so that every
-// MFMA operand is one 16-byte LDS read.  After each round of 8 units the
-// wavefronts fold their (m, l, R*v2) into the workgroup's fp32 accumulator
-// through bf16 slabs in LDS, each thread summing a fixed slice in a fixed order.
+// window [i0-w1, i0+31] in 32-key tiles that the workgroup stages through a
+// three-deep LDS ring: K row-major, V transposed and permuted so that every
+// MFMA operand is one 16-byte LDS read.  The q rows of the block and the K'/V'
+// rows its deltas reach are copied to LDS once.  On unmasked tiles wavefronts
+// 4-7 run their value MFMAs one tile late, so that on each SIMD one wavefront's
+// softmax arithmetic coincides with the other's MFMAs although all eight meet at
+// one barrier per tile.  After each round of 8 units the wavefronts fold their
+// (m, l, R*v2) into the workgroup's fp32 accumulator through bf16 slabs in LDS,
+// each thread summing a fixed slice in a fixed order.
 //
 // The logits are computed transposed (S^T = K1 . Q~^T) so that an expanded row
 // lives in one lane pair: exp2(S^T) is already laid out as the B operand of
@@ -46,11 +50,18 @@ struct Cfg {
     static constexpr int SS = D + 8;                        // slab row stride (bf16)
     static constexpr int OS = D + 4;                        // accumulator row stride (fp32)
     // LDS carve-up (bytes)
-    static constexpr size_t STAGE_BYTES = (size_t)2 * STAGE * 2;
-    static constexpr size_t SLAB_BYTES = (size_t)FW * BQ * SS * 2;
+    static constexpr int NSTAGE = 3;
+    static constexpr size_t STAGE_BYTES = (size_t)NSTAGE * STAGE * 2;
+    static constexpr size_t SLAB_BYTES = (size_t)4 * BQ * SS * 2;          // two sets of two slabs
     static constexpr size_t OACC_BYTES = (size_t)BQ * OS * 4;
     static constexpr size_t XCH_BYTES = (size_t)(2 * FW * BQ + 3 * BQ) * 4;
-    static constexpr size_t LDS_BYTES = STAGE_BYTES + SLAB_BYTES + OACC_BYTES + XCH_BYTES;
+    static constexpr size_t QS_BYTES = (size_t)BQ * KS * 2;
+    static constexpr size_t BASE_BYTES = STAGE_BYTES + SLAB_BYTES + OACC_BYTES + XCH_BYTES + QS_BYTES;
+    static constexpr size_t LDS_LIMIT = 160 * 1024;
+    // rows of K' and V' kept in LDS: the 32 of the block plus the w2 before it
+    static size_t side_bytes(int w2) { return (size_t)2 * (BQ + w2) * KS * 2; }
+    static bool side_fits(int w2) { return BASE_BYTES + side_bytes(w2) <= LDS_LIMIT; }
+    static size_t lds_bytes(int w2) { return BASE_BYTES + (side_fits(w2) ? side_bytes(w2) : 0); }
 };
 
 // SAFE = false: the fast kernel.  A weight that overflows (logits growing by more
@@ -61,7 +72,7 @@ struct Cfg {
 // exits at once.
 template <int D, bool SAFE>
 __global__ __launch_bounds__(FT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_fwd_kernel(Problem p, int nqb, int total) {
+void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* smem = (uint16_t*)smem_raw;
@@ -72,6 +83,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     float* xch_a = xch_l + FW * BQ;             // [BQ] accumulator rescale of this round
     float* fin_m = xch_a + BQ;                  // [BQ] final M
     float* fin_l = fin_m + BQ;                  // [BQ] final L
+    uint16_t* q_s = (uint16_t*)(fin_l + BQ);    // [BQ][KS] q rows of the block
+    uint16_t* k2_s = q_s + BQ * C::KS;          // [BQ + w2][KS] K' rows i0-w2 .. i0+31 (when side_kv)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -172,6 +185,37 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     float Mrun = -INFINITY, Lrun = 0.f;            // per query (lane), replicated in every wavefront
     bool bad = false;
 
+    // ---- q rows of the block and the K'/V' rows its deltas reach, once, to LDS ----
+    const int side_rows = BQ + w2;
+    uint16_t* v2_s = k2_s + side_rows * C::KS;
+    {
+        constexpr int CPR = D / 8;                 // 16-byte chunks per row
+        for (int c = tid; c < BQ * CPR; c += FT) {
+            const int row = c / CPR, col = c - row * CPR;
+            int r = i0 + row;
+            r = r < N ? r : N - 1;
+            *(uint4*)(q_s + row * C::KS + col * 8) = *(const uint4*)(qp + (int64_t)r * p.q.sn + col * 8);
+        }
+        if (side_kv) {
+            for (int c = tid; c < side_rows * CPR; c += FT) {
+                const int row = c / CPR, col = c - row * CPR;
+                int r = i0 - w2 + row;
+                r = r < 0 ? 0 : (r < N ? r : N - 1);
+                *(uint4*)(k2_s + row * C::KS + col * 8) = *(const uint4*)(k2p + (int64_t)r * p.k2.sn + col * 8);
+                *(uint4*)(v2_s + row * C::KS + col * 8) = *(const uint4*)(v2p + (int64_t)r * p.v2.sn + col * 8);
+            }
+        }
+    }
+    // K'/V' row of this lane's query for a given delta: LDS copy or global memory
+    const uint16_t* k2src = side_kv ? (const uint16_t*)k2_s : k2p;
+    const uint16_t* v2src = side_kv ? (const uint16_t*)v2_s : v2p;
+    const int64_t k2stride = side_kv ? C::KS : p.k2.sn, v2stride = side_kv ? C::KS : p.v2.sn;
+    auto side_row = [&](int delta) {
+        if (side_kv) return ln + w2 - delta;       // (i0 + ln - delta) - (i0 - w2)
+        int k = ic - delta;
+        return k > 0 ? k : 0;
+    };
+
     const float qscale = p.scale * LOG2E;
 
     load_tile(jt_lo);
@@ -184,12 +228,25 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
     int s_lo = (i0 + BQ - 1 - w1 + TJ - 1) / TJ - jt_lo;       // first tile with j0 >= i0+31-w1
     s_lo = (i0 + BQ - 1 - w1 <= jt_lo * TJ) ? 0 : s_lo;
     const int s_hi = (i0 + 1) / TJ - 1 - jt_lo;                 // last tile with j0+31 <= i0
+    const bool late_values = wave >= FW / 2;                    // wavefronts 4-7: value MFMAs one tile late
 
-    int g = 0;
+    int g = 0, buf = 0;                                         // buf = g % NSTAGE
+    auto advance = [&]() {
+        // end of a tile step: next tile to LDS, the one after to registers, barrier
+        const int nb = buf + 1 == C::NSTAGE ? 0 : buf + 1;
+        if (g + 1 < total_steps) store_tile(nb);
+        if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
+        __syncthreads();
+        buf = nb;
+        ++g;
+    };
+
     for (int round = 0; round < nrounds; ++round) {
         const int delta = round * FW + wave;
         const bool ok = delta < n_units;
-        float m = -INFINITY, l = 0.f;
+        // The unit starts from the query's running reference point (finite from the second
+        // round on), so only the first round has to look for maxima.
+        float m = ok ? Mrun : -INFINITY, l = 0.f;
         floatx16 racc[C::DT];
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
@@ -198,21 +255,17 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
 
         if (!ok) {
             // no unit for this wavefront in this round: keep the staging pipeline moving
-            for (int s = 0; s < nt; ++s, ++g) {
-                if (g + 1 < total_steps) store_tile((g + 1) & 1);
-                if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
-                __syncthreads();
-            }
+            for (int s = 0; s < nt; ++s) advance();
         } else {
             // ---- new unit: Q~ operand, fresh softmax state ----------------------
             bf16x8 qf[C::DK];
             {
-                int k = ic - delta;
-                k = k > 0 ? k : 0;
+                const uint16_t* krow = k2src + (int64_t)side_row(delta) * k2stride + hf * 8;
+                const uint16_t* qrow = q_s + ln * C::KS + hf * 8;
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
-                    const uint4 qa = *(const uint4*)(qp + (int64_t)ic * p.q.sn + kk * 16 + hf * 8);
-                    const uint4 kb = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + kk * 16 + hf * 8);
+                    const uint4 qa = *(const uint4*)(qrow + kk * 16);
+                    const uint4 kb = *(const uint4*)(krow + kk * 16);
                     const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
                     const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
                     bf16x8 r;
@@ -228,10 +281,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
             const bool row_ok = i < N && i >= delta;
             // -m (0 while the row has no finite logit yet), as a scalar and replicated over an
             // accumulator tuple: the tuple is the C operand of the first logit MFMA.
-            float nm = 0.f;
+            float nm = (m == -INFINITY) ? 0.f : -m;
             floatx16 negm;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) negm[v] = 0.f;
+            for (int v = 0; v < 16; ++v) negm[v] = nm;
 
             // exp2 of the shifted logits -> bf16 weights (MFMA B operand) and their row sum
             auto weights = [&](const floatx16& sh, bf16x8* w, float& rsum) {
@@ -249,6 +302,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                     r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 6, 7), ones, r, false);
                 }
                 rsum = r;
+            };
+            auto logit_mfmas = [&](const uint16_t* Ks, floatx16 c) -> floatx16 {
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) {
+                    const bf16x8 ka = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], c, 0, 0, 0);
+                }
+                return c;
             };
             auto value_mfmas = [&](const uint16_t* Vt, const bf16x8* w) {
 #pragma unroll
@@ -268,21 +329,16 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                 if (s < fast_lo || s >= fast_hi) {
                     // ---- general tile: masks, and a (new) reference point where needed ----
                     const int j0 = (jt_lo + s) * TJ;
-                    const uint16_t* Ks = smem + (g & 1) * C::STAGE;
+                    const uint16_t* Ks = smem + buf * C::STAGE;
                     const uint16_t* Vt = Ks + C::K_ELEMS;
                     const bool plain = (j0 + TJ - 1 <= i0) && (j0 >= i0 + BQ - 1 - w1) && rows_full;
                     // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
                     const int hi = i - j0 - 4 * hf, lo = hi - w1;
-                    bf16x8 ka[C::DK];
-#pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
-                    if (SAFE || s == 0 || __builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
+                    if (SAFE || __builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
                         floatx16 t;
 #pragma unroll
                         for (int v = 0; v < 16; ++v) t[v] = 0.f;
-#pragma unroll
-                        for (int kk = 0; kk < C::DK; ++kk)
-                            t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], t, 0, 0, 0);
+                        t = logit_mfmas(Ks, t);
                         float mx = -INFINITY;
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
@@ -298,12 +354,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                             const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
                             m = m_new;
                             l *= alpha;
-                            if (s > 0) {
 #pragma unroll
-                                for (int dt = 0; dt < C::DT; ++dt)
+                            for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                                    for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
-                            }
+                                for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
                             nm = (m_new == -INFINITY) ? 0.f : -m_new;
 #pragma unroll
                             for (int v = 0; v < 16; ++v) negm[v] = nm;
@@ -316,41 +370,49 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                         const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
                         ct[v] = valid ? nm : -INFINITY;
                     }
-#pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk)
-                        ct = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], ct, 0, 0, 0);
+                    ct = logit_mfmas(Ks, ct);
                     bf16x8 pb[2];
                     float rs;
                     weights(ct, pb, rs);
                     l += rs;
                     bad |= !(rs < OVERFLOW_LIMIT);
                     value_mfmas(Vt, pb);
-                    if (g + 1 < total_steps) store_tile((g + 1) & 1);
-                    if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
-                    __syncthreads();
+                    advance();
                     ++s;
-                    ++g;
                     continue;
                 }
                 // ---- unmasked tiles: reference point fixed, straight-line body ----
-                for (; s < fast_hi; ++s, ++g) {
-                    const uint16_t* Ks = smem + (g & 1) * C::STAGE;
-                    const uint16_t* Vt = Ks + C::K_ELEMS;
-                    floatx16 sh = negm;
-#pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) {
-                        const bf16x8 ka = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], sh, 0, 0, 0);
+                if (!late_values) {
+                    for (; s < fast_hi; ++s) {
+                        const uint16_t* Ks = smem + buf * C::STAGE;
+                        bf16x8 pb[2];
+                        float rs;
+                        weights(logit_mfmas(Ks, negm), pb, rs);
+                        l += rs;
+                        bad |= !(rs < OVERFLOW_LIMIT);
+                        value_mfmas(Ks + C::K_ELEMS, pb);
+                        advance();
                     }
+                } else {
+                    // same work, value MFMAs of tile t issued at the start of tile t+1
                     bf16x8 pb[2];
                     float rs;
-                    weights(sh, pb, rs);
+                    const uint16_t* Vt_prev = smem + buf * C::STAGE + C::K_ELEMS;
+                    weights(logit_mfmas(smem + buf * C::STAGE, negm), pb, rs);
                     l += rs;
                     bad |= !(rs < OVERFLOW_LIMIT);
-                    value_mfmas(Vt, pb);
-                    if (g + 1 < total_steps) store_tile((g + 1) & 1);
-                    if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
-                    __syncthreads();
+                    advance();
+                    ++s;
+                    for (; s < fast_hi; ++s) {
+                        const uint16_t* Ks = smem + buf * C::STAGE;
+                        value_mfmas(Vt_prev, pb);
+                        Vt_prev = Ks + C::K_ELEMS;
+                        weights(logit_mfmas(Ks, negm), pb, rs);
+                        l += rs;
+                        bad |= !(rs < OVERFLOW_LIMIT);
+                        advance();
+                    }
+                    value_mfmas(Vt_prev, pb);
                 }
             }
         }
@@ -373,37 +435,37 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
         Mrun = Mn;
         Lrun = Ln;
         if (wave == 0 && hf == 0) xch_a[ln] = a;
-        {
-            // this wavefront's contribution, bf16, to its slab: c * (v2 + bias) * R
-            const float cw = ok ? fast_exp2(m - Muse) : 0.f;
-            int kr = ic - delta;
-            kr = kr > 0 ? kr : 0;
-            const uint16_t* vrow = v2p + (int64_t)kr * p.v2.sn + 4 * hf;
-            uint16_t* srow = slabs + (wave * BQ + ln) * C::SS + 4 * hf;
+        const float cw = ok ? fast_exp2(m - Muse) : 0.f;
+        const uint16_t* vrow = v2src + (int64_t)(ok ? side_row(delta) : 0) * v2stride + 4 * hf;
+        float acc[ACN];
+        // four phases of two wavefronts: contribution c * (v2 + bias) * R as bf16 into a slab
+        // (two slab sets alternate), then every thread adds its slice in wavefront order
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt)
+        for (int ph = 0; ph < FW / 2; ++ph) {
+            if ((wave >> 1) == ph) {
+                uint16_t* srow = slabs + (((ph & 1) * 2 + (wave & 1)) * BQ + ln) * C::SS + 4 * hf;
 #pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    uint2 x = make_uint2(0u, 0u);
-                    if (ok) x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
-                    union { __bf16 h[4]; uint2 u; } o;
-                    o.h[0] = (__bf16)(cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
-                    o.h[1] = (__bf16)(cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
-                    o.h[2] = (__bf16)(cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
-                    o.h[3] = (__bf16)(cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
-                    *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
-                }
-        }
-        __syncthreads();
-        {
-            // each thread sums its slice of the 8 slabs in wavefront order
-            const float ar = xch_a[aq];
-            float acc[ACN];
+                for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-            for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c] * ar;
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        union { __bf16 h[4]; uint2 u; } o;
+                        o.h[0] = (__bf16)(cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
+                        o.h[1] = (__bf16)(cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
+                        o.h[2] = (__bf16)(cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
+                        o.h[3] = (__bf16)(cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
+                        *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
+                    }
+            }
+            __syncthreads();
+            if (ph == 0) {
+                const float ar = xch_a[aq];
 #pragma unroll
-            for (int w = 0; w < FW; ++w) {
-                const uint16_t* sp = slabs + (w * BQ + aq) * C::SS + ac;
+                for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c] * ar;
+            }
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+                const uint16_t* sp = slabs + (((ph & 1) * 2 + w) * BQ + aq) * C::SS + ac;
                 if (ACN == 8) {
                     const uint4 x = *(const uint4*)sp;
                     acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
@@ -414,10 +476,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
                     acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
                 }
             }
-#pragma unroll
-            for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
         }
-        // (the slabs and exchange arrays are next written a whole tile sweep of barriers later)
+#pragma unroll
+        for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
+        // (slabs and exchange arrays are next written a whole tile sweep of barriers later)
     }
 
     // ---- normalise and store ------------------------------------------------------
@@ -449,14 +511,16 @@ void mfma_fwd_kernel(Problem p, int nqb, int total) {
 template <int D>
 int launch_fwd_pair(const Problem& p, int nqb, int total, hipStream_t st) {
     using C = Cfg<D>;
+    const int side_kv = C::side_fits(p.w2) ? 1 : 0;
+    const size_t lds = C::lds_bytes(p.w2);
     if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)C::LDS_BYTES) != hipSuccess ||
+                            (int)lds) != hipSuccess ||
         hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)C::LDS_BYTES) != hipSuccess)
+                            (int)lds) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL((mfma_fwd_kernel<D, false>), dim3((unsigned)total), dim3(FT), C::LDS_BYTES, st, p, nqb, total);
+    hipLaunchKernelGGL((mfma_fwd_kernel<D, false>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, side_kv);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL((mfma_fwd_kernel<D, true>), dim3((unsigned)total), dim3(FT), C::LDS_BYTES, st, p, nqb, total);
+    hipLaunchKernelGGL((mfma_fwd_kernel<D, true>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, side_kv);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
 
