@@ -16,10 +16,10 @@
 // window [i0-w1, i0+31] in 32-key tiles that the workgroup stages through a
 // three-deep LDS ring: K row-major, V transposed and permuted so that every
 // MFMA operand is one 16-byte LDS read.  The q rows of the block and the K'/V'
-// rows its deltas reach are copied to LDS once.  On unmasked tiles wavefronts
-// 4-7 run their value MFMAs one tile late, so that on each SIMD one wavefront's
-// softmax arithmetic coincides with the other's MFMAs although all eight meet at
-// one barrier per tile.  After each round of 8 units the wavefronts fold their
+// rows its deltas reach are copied to LDS once.  On unmasked tiles each step
+// issues the logit MFMAs of tile t between the softmax instructions of tile t-1
+// and then the value MFMAs of tile t-1, so neither pipe waits for the other inside
+// the one barrier interval per tile.  After each round of 8 units the wavefronts fold their
 // (m, l, R*v2) into the workgroup's fp32 accumulator through bf16 slabs in LDS,
 // each thread summing a fixed slice in a fixed order.
 //
@@ -228,7 +228,6 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     int s_lo = (i0 + BQ - 1 - w1 + TJ - 1) / TJ - jt_lo;       // first tile with j0 >= i0+31-w1
     s_lo = (i0 + BQ - 1 - w1 <= jt_lo * TJ) ? 0 : s_lo;
     const int s_hi = (i0 + 1) / TJ - 1 - jt_lo;                 // last tile with j0+31 <= i0
-    const bool late_values = wave >= FW / 2;                    // wavefronts 4-7: value MFMAs one tile late
 
     int g = 0, buf = 0;                                         // buf = g % NSTAGE
     auto advance = [&]() {
@@ -381,37 +380,38 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     ++s;
                     continue;
                 }
-                // ---- unmasked tiles: reference point fixed, straight-line body ----
-                if (!late_values) {
-                    for (; s < fast_hi; ++s) {
-                        const uint16_t* Ks = smem + buf * C::STAGE;
-                        bf16x8 pb[2];
-                        float rs;
-                        weights(logit_mfmas(Ks, negm), pb, rs);
-                        l += rs;
-                        bad |= !(rs < OVERFLOW_LIMIT);
-                        value_mfmas(Ks + C::K_ELEMS, pb);
-                        advance();
-                    }
-                } else {
-                    // same work, value MFMAs of tile t issued at the start of tile t+1
-                    bf16x8 pb[2];
-                    float rs;
+                // ---- unmasked tiles: reference point fixed, two-stage software pipeline ----
+                // Step t issues the logit MFMAs of tile t interleaved with the softmax
+                // arithmetic of tile t-1 (independent streams), then the value MFMAs of
+                // tile t-1; the shifted logits of tile t wait in registers for step t+1.
+                {
+                    floatx16 sh_prev = logit_mfmas(smem + buf * C::STAGE, negm);
                     const uint16_t* Vt_prev = smem + buf * C::STAGE + C::K_ELEMS;
-                    weights(logit_mfmas(smem + buf * C::STAGE, negm), pb, rs);
-                    l += rs;
-                    bad |= !(rs < OVERFLOW_LIMIT);
                     advance();
                     ++s;
                     for (; s < fast_hi; ++s) {
                         const uint16_t* Ks = smem + buf * C::STAGE;
-                        value_mfmas(Vt_prev, pb);
-                        Vt_prev = Ks + C::K_ELEMS;
-                        weights(logit_mfmas(Ks, negm), pb, rs);
+                        bf16x8 pb[2];
+                        float rs;
+                        const floatx16 sh = logit_mfmas(Ks, negm);
+                        weights(sh_prev, pb, rs);
                         l += rs;
                         bad |= !(rs < OVERFLOW_LIMIT);
+                        value_mfmas(Vt_prev, pb);
+#pragma unroll
+                        for (int x = 0; x < C::DK; ++x) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x402, 48 / C::DK, 0);      // a slice of VALU / exp
+                        }
+                        sh_prev = sh;
+                        Vt_prev = Ks + C::K_ELEMS;
                         advance();
                     }
+                    bf16x8 pb[2];
+                    float rs;
+                    weights(sh_prev, pb, rs);
+                    l += rs;
+                    bad |= !(rs < OVERFLOW_LIMIT);
                     value_mfmas(Vt_prev, pb);
                 }
             }
