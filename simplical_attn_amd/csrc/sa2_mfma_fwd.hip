@@ -391,13 +391,31 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     ++s;
                     for (; s < fast_hi; ++s) {
                         const uint16_t* Ks = smem + buf * C::STAGE;
+                        // all sixteen operand reads of the step go out first: the LDS latency is
+                        // paid once, not once per MFMA
+                        bf16x8 ka[C::DK], va[C::DT][2];
+#pragma unroll
+                        for (int kk = 0; kk < C::DK; ++kk) ka[kk] = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+#pragma unroll
+                        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                            for (int ks = 0; ks < 2; ++ks)
+                                va[dt][ks] = *(const bf16x8*)(Vt_prev + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
                         bf16x8 pb[2];
                         float rs;
-                        const floatx16 sh = logit_mfmas(Ks, negm);
+                        floatx16 sh = negm;
+#pragma unroll
+                        for (int kk = 0; kk < C::DK; ++kk)
+                            sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sh, 0, 0, 0);
                         weights(sh_prev, pb, rs);
                         l += rs;
                         bad |= !(rs < OVERFLOW_LIMIT);
-                        value_mfmas(Vt_prev, pb);
+#pragma unroll
+                        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                            for (int ks = 0; ks < 2; ++ks)
+                                racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, C::DK + 2 * C::DT, 0);       // the LDS reads
 #pragma unroll
                         for (int x = 0; x < C::DK; ++x) {
                             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
