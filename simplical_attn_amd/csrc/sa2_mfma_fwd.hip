@@ -280,7 +280,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
             const bool row_ok = i < N && i >= delta;
             // -m (0 while the row has no finite logit yet), as a scalar and replicated over an
             // accumulator tuple: the tuple is the C operand of the first logit MFMA.
-            float nm = (m == -INFINITY) ? 0.f : -m;
+            float nm = (m == -INFINITY) ? 0.f : -m;    // (first round: fixed before the sweep)
             floatx16 negm;
 #pragma unroll
             for (int v = 0; v < 16; ++v) negm[v] = nm;
@@ -320,118 +320,139 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     }
             };
 
-            const int fast_lo = (!SAFE && rows_full) ? (s_lo > 1 ? s_lo : 1) : nt;
-            const int fast_hi = (!SAFE && rows_full) ? s_hi + 1 : nt;   // exclusive
+            // Mask of a tile as the C operand of its logit MFMAs: -m where the key is inside
+            // the window of the row, -inf elsewhere.  Element v of this lane is key
+            // j0 + 8*(v/4) + 4*hf + v%4.
+            auto masked_c = [&](int j0) -> floatx16 {
+                const int hi = i - j0 - 4 * hf, lo = hi - w1;
+                floatx16 ct;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int c = 8 * (v >> 2) + (v & 3);
+                    const bool valid = row_ok & (c <= hi) & (c >= lo);
+                    ct[v] = valid ? nm : -INFINITY;
+                }
+                return ct;
+            };
+            auto tile_plain = [&](int s) {
+                return rows_full && s >= s_lo && s <= s_hi;
+            };
 
-            int s = 0;
-            while (s < nt) {
-                if (s < fast_lo || s >= fast_hi) {
-                    // ---- general tile: masks, and a (new) reference point where needed ----
+            if (SAFE) {
+                // ---- repair pass: the reference point follows the maxima on every tile ----
+                for (int s = 0; s < nt; ++s) {
                     const int j0 = (jt_lo + s) * TJ;
                     const uint16_t* Ks = smem + buf * C::STAGE;
-                    const uint16_t* Vt = Ks + C::K_ELEMS;
-                    const bool plain = (j0 + TJ - 1 <= i0) && (j0 >= i0 + BQ - 1 - w1) && rows_full;
-                    // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
+                    const bool plain = tile_plain(s);
                     const int hi = i - j0 - 4 * hf, lo = hi - w1;
-                    if (SAFE || __builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
-                        floatx16 t;
+                    floatx16 t;
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) t[v] = 0.f;
-                        t = logit_mfmas(Ks, t);
-                        float mx = -INFINITY;
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int c = 8 * (v >> 2) + (v & 3);
-                            const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
-                            mx = fmaxf(mx, valid ? t[v] : -INFINITY);
-                        }
-                        mx = fmaxf(mx, other_half(mx));
-                        // Lazy: move the reference only when the maximum grew by more than
-                        // 2^RESCALE_LOG2; later formulas only need m as a common reference.
-                        const float m_new = (mx > m + RESCALE_LOG2) ? mx : m;
-                        if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
-                            const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
-                            m = m_new;
-                            l *= alpha;
-#pragma unroll
-                            for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                                for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
-                            nm = (m_new == -INFINITY) ? 0.f : -m_new;
-#pragma unroll
-                            for (int v = 0; v < 16; ++v) negm[v] = nm;
-                        }
-                    }
-                    floatx16 ct;
+                    for (int v = 0; v < 16; ++v) t[v] = 0.f;
+                    t = logit_mfmas(Ks, t);
+                    float mx = -INFINITY;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int c = 8 * (v >> 2) + (v & 3);
                         const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
-                        ct[v] = valid ? nm : -INFINITY;
+                        t[v] = valid ? t[v] : -INFINITY;
+                        mx = fmaxf(mx, t[v]);
                     }
-                    ct = logit_mfmas(Ks, ct);
+                    mx = fmaxf(mx, other_half(mx));
+                    const float m_new = fmaxf(m, mx);
+                    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                    const float alpha = fast_exp2(m - m_use);
+                    m = m_new;
+                    l *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) t[v] -= m_use;
                     bf16x8 pb[2];
                     float rs;
-                    weights(ct, pb, rs);
+                    weights(t, pb, rs);
                     l += rs;
-                    bad |= !(rs < OVERFLOW_LIMIT);
-                    value_mfmas(Vt, pb);
+                    value_mfmas(Ks + C::K_ELEMS, pb);
                     advance();
-                    ++s;
-                    continue;
                 }
-                // ---- unmasked tiles: reference point fixed, two-stage software pipeline ----
-                // Step t issues the logit MFMAs of tile t interleaved with the softmax
-                // arithmetic of tile t-1 (independent streams), then the value MFMAs of
-                // tile t-1; the shifted logits of tile t wait in registers for step t+1.
-                {
-                    floatx16 sh_prev = logit_mfmas(smem + buf * C::STAGE, negm);
-                    const uint16_t* Vt_prev = smem + buf * C::STAGE + C::K_ELEMS;
-                    advance();
-                    ++s;
-                    for (; s < fast_hi; ++s) {
-                        const uint16_t* Ks = smem + buf * C::STAGE;
-                        // all sixteen operand reads of the step go out first: the LDS latency is
-                        // paid once, not once per MFMA
-                        bf16x8 ka[C::DK], va[C::DT][2];
+            } else {
+                // ---- reference point: the query's running one, or (first round) the maximum of
+                // the first tile, or 0 for a row with no key there.  Any finite reference is
+                // exact as long as no weight overflows, which `bad` watches.
+                if (__builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
+                    const int j0 = jt_lo * TJ;
+                    const int hi = i - j0 - 4 * hf, lo = hi - w1;
+                    floatx16 t;
 #pragma unroll
-                        for (int kk = 0; kk < C::DK; ++kk) ka[kk] = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+                    for (int v = 0; v < 16; ++v) t[v] = 0.f;
+                    t = logit_mfmas(smem + buf * C::STAGE, t);
+                    float mx = -INFINITY;
 #pragma unroll
-                        for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                            for (int ks = 0; ks < 2; ++ks)
-                                va[dt][ks] = *(const bf16x8*)(Vt_prev + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
-                        bf16x8 pb[2];
-                        float rs;
-                        floatx16 sh = negm;
-#pragma unroll
-                        for (int kk = 0; kk < C::DK; ++kk)
-                            sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sh, 0, 0, 0);
-                        weights(sh_prev, pb, rs);
-                        l += rs;
-                        bad |= !(rs < OVERFLOW_LIMIT);
-#pragma unroll
-                        for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                            for (int ks = 0; ks < 2; ++ks)
-                                racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x100, C::DK + 2 * C::DT, 0);       // the LDS reads
-#pragma unroll
-                        for (int x = 0; x < C::DK; ++x) {
-                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
-                            __builtin_amdgcn_sched_group_barrier(0x402, 48 / C::DK, 0);      // a slice of VALU / exp
-                        }
-                        sh_prev = sh;
-                        Vt_prev = Ks + C::K_ELEMS;
-                        advance();
+                    for (int v = 0; v < 16; ++v) {
+                        const int c = 8 * (v >> 2) + (v & 3);
+                        const bool valid = row_ok & (c <= hi) & (c >= lo);
+                        mx = fmaxf(mx, valid ? t[v] : -INFINITY);
                     }
+                    mx = fmaxf(mx, other_half(mx));
+                    if (m == -INFINITY) m = (mx == -INFINITY) ? 0.f : mx;
+                    nm = -m;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) negm[v] = nm;
+                }
+                // ---- two-stage software pipeline over the tiles: step t issues the logit MFMAs
+                // of tile t between the softmax instructions of tile t-1, then the value MFMAs
+                // of tile t-1; the shifted logits of tile t wait in registers for step t+1.
+                floatx16 sh_prev;
+                {
+                    const floatx16 c0 = tile_plain(0) ? negm : masked_c(jt_lo * TJ);
+                    sh_prev = logit_mfmas(smem + buf * C::STAGE, c0);
+                }
+                const uint16_t* Vt_prev = smem + buf * C::STAGE + C::K_ELEMS;
+                advance();
+                for (int s = 1; s < nt; ++s) {
+                    const uint16_t* Ks = smem + buf * C::STAGE;
+                    // all sixteen operand reads of the step go out first: the LDS latency is
+                    // paid once, not once per MFMA
+                    bf16x8 ka[C::DK], va[C::DT][2];
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks)
+                            va[dt][ks] = *(const bf16x8*)(Vt_prev + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                    floatx16 sh = negm;
+                    if (__builtin_expect(!tile_plain(s), 0)) sh = masked_c((jt_lo + s) * TJ);
                     bf16x8 pb[2];
                     float rs;
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk)
+                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sh, 0, 0, 0);
                     weights(sh_prev, pb, rs);
                     l += rs;
                     bad |= !(rs < OVERFLOW_LIMIT);
-                    value_mfmas(Vt_prev, pb);
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks)
+                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK + 2 * C::DT, 0);       // the LDS reads
+#pragma unroll
+                    for (int x = 0; x < C::DK; ++x) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x402, 48 / C::DK, 0);      // a slice of VALU / exp
+                    }
+                    sh_prev = sh;
+                    Vt_prev = Ks + C::K_ELEMS;
+                    advance();
                 }
+                bf16x8 pb[2];
+                float rs;
+                weights(sh_prev, pb, rs);
+                l += rs;
+                bad |= !(rs < OVERFLOW_LIMIT);
+                value_mfmas(Vt_prev, pb);
             }
         }
 
