@@ -52,7 +52,8 @@ struct Cfg {
     // LDS carve-up (bytes)
     static constexpr int NSTAGE = 3;
     static constexpr size_t STAGE_BYTES = (size_t)NSTAGE * STAGE * 2;
-    static constexpr size_t SLAB_BYTES = (size_t)4 * BQ * SS * 2;          // two sets of two slabs
+    static constexpr size_t SLAB_BYTES = (size_t)4 * BQ * SS * 2;          // four slabs; four more live in idle stage buffers
+    static_assert(2 * BQ * SS <= STAGE, "two slabs must fit one stage buffer");
     static constexpr size_t OACC_BYTES = (size_t)BQ * OS * 4;
     static constexpr size_t XCH_BYTES = (size_t)(2 * FW * BQ + 3 * BQ) * 4;
     static constexpr size_t QS_BYTES = (size_t)BQ * KS * 2;
@@ -474,37 +475,42 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         Mrun = Mn;
         Lrun = Ln;
         if (wave == 0 && hf == 0) xch_a[ln] = a;
+        // Every wavefront writes its contribution c * (v2 + bias) * R as bf16 into its own
+        // slab: four slabs have their own LDS, the other four use the two stage buffers
+        // that hold no live tile between rounds.  Then every thread adds its slice of the
+        // eight slabs in wavefront order.
         const float cw = ok ? fast_exp2(m - Muse) : 0.f;
         const uint16_t* vrow = v2src + (int64_t)(ok ? side_row(delta) : 0) * v2stride + 4 * hf;
-        float acc[ACN];
-        // four phases of two wavefronts: contribution c * (v2 + bias) * R as bf16 into a slab
-        // (two slab sets alternate), then every thread adds its slice in wavefront order
+        auto slab_of = [&](int w) -> uint16_t* {
+            if (w < 4) return slabs + w * (BQ * C::SS);
+            int fb = buf + 1 + ((w - 4) >> 1);                 // the two stage buffers other than buf
+            fb = fb >= C::NSTAGE ? fb - C::NSTAGE : fb;
+            return smem + fb * C::STAGE + ((w - 4) & 1) * (BQ * C::SS);
+        };
+        {
+            uint16_t* srow = slab_of(wave) + ln * C::SS + 4 * hf;
 #pragma unroll
-        for (int ph = 0; ph < FW / 2; ++ph) {
-            if ((wave >> 1) == ph) {
-                uint16_t* srow = slabs + (((ph & 1) * 2 + (wave & 1)) * BQ + ln) * C::SS + 4 * hf;
+            for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt)
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                    union { __bf16 h[4]; uint2 u; } o;
+                    o.h[0] = (__bf16)(cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
+                    o.h[1] = (__bf16)(cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
+                    o.h[2] = (__bf16)(cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
+                    o.h[3] = (__bf16)(cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
+                    *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
+                }
+        }
+        __syncthreads();
+        {
+            const float ar = xch_a[aq];
+            float acc[ACN];
 #pragma unroll
-                    for (int g4 = 0; g4 < 4; ++g4) {
-                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
-                        union { __bf16 h[4]; uint2 u; } o;
-                        o.h[0] = (__bf16)(cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
-                        o.h[1] = (__bf16)(cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
-                        o.h[2] = (__bf16)(cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
-                        o.h[3] = (__bf16)(cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
-                        *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
-                    }
-            }
-            __syncthreads();
-            if (ph == 0) {
-                const float ar = xch_a[aq];
+            for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c] * ar;
 #pragma unroll
-                for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c] * ar;
-            }
-#pragma unroll
-            for (int w = 0; w < 2; ++w) {
-                const uint16_t* sp = slabs + (((ph & 1) * 2 + w) * BQ + aq) * C::SS + ac;
+            for (int w = 0; w < FW; ++w) {
+                const uint16_t* sp = slab_of(w) + aq * C::SS + ac;
                 if (ACN == 8) {
                     const uint4 x = *(const uint4*)sp;
                     acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
@@ -515,10 +521,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
                 }
             }
-        }
 #pragma unroll
-        for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
-        // (slabs and exchange arrays are next written a whole tile sweep of barriers later)
+            for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
+        }
+        __syncthreads();       // the stage buffers that served as slabs are written again by the next step
     }
 
     // ---- normalise and store ------------------------------------------------------
