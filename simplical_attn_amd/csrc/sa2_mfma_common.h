@@ -32,6 +32,27 @@ __device__ __forceinline__ float other_half(float x) {
     return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
 }
 
+// Eight bf16 of one COLUMN of a row-major [row][col] bf16 tile in LDS, as the A/B operand
+// of a 32x32x16 MFMA whose contraction index runs over the tile's rows.  `tile` points at
+// the tile's 32x32 sub-block (rows r0.., columns c0..), `stride` is the row stride in
+// elements.  Lane l gets column c0 + l%32 and, for its half h = l/32, the rows
+//   r0 + 16*ks + 4*h + {0,1,2,3}   and   r0 + 16*ks + 8 + 4*h + {0,1,2,3}
+// which is exactly the k-slot order in which a 32x32 accumulator tile (rows = those rows)
+// hands its values to the other operand.  Uses the LDS transpose read: within 16 lanes,
+// lane s supplies the address of row s/4, columns 4*(s%4)..+3, and lane i receives
+// column i of those four rows.
+__device__ __forceinline__ bf16x8 lds_column_operand(const uint16_t* tile, int stride, int ks, int lane) {
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    const int grp = lane >> 4, s = lane & 15;
+    const uint16_t* p0 = tile + (16 * ks + 4 * (grp >> 1) + (s >> 2)) * stride + 16 * (grp & 1) + 4 * (s & 3);
+    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)p0);
+    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(p0 + 8 * stride));
+    union { v4s h[2]; bf16x8 v; } u;
+    u.h[0] = a;
+    u.h[1] = b;
+    return u.v;
+}
+
 // acc *= alpha for an MFMA accumulator that lives in AGPRs, without asking the
 // register allocator for a VGPR copy of the tuple (it would place that copy on
 // the hot path).  Used only on the rare rescale path; the s_nop before the

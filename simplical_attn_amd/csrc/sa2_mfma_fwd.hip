@@ -14,8 +14,8 @@
 // queries of one (batch, head).  A "unit" is (delta, those 32 queries) = one
 // 32-row MFMA N-tile; each wavefront holds one unit at a time and sweeps the K
 // window [i0-w1, i0+31] in 32-key tiles that the workgroup stages through a
-// three-deep LDS ring: K row-major, V transposed and permuted so that every
-// MFMA operand is one 16-byte LDS read.  The q rows of the block and the K'/V'
+// three-deep LDS ring, both row-major; K operands are 16-byte LDS reads, V
+// operands come out of LDS transposed (ds_read_b64_tr_b16).  The q rows of the block and the K'/V'
 // rows its deltas reach are copied to LDS once.  On unmasked tiles each step
 // issues the logit MFMAs of tile t between the softmax instructions of tile t-1
 // and then the value MFMAs of tile t-1, so neither pipe waits for the other inside
@@ -41,12 +41,11 @@ struct Cfg {
     static constexpr int DK = D / 16;          // k-steps of the logit contraction
     static constexpr int DT = D / 32;          // 32-column tiles of the value contraction
     static constexpr int KS = D + 8;           // K tile row stride in LDS (bf16), +16 B against bank conflicts
-    static constexpr int VS = TJ + 8;          // V^T tile row stride in LDS (bf16)
+    static constexpr int VS = D + 16;          // V tile row stride in LDS (bf16), +32 B: conflict-free transpose reads
     static constexpr int K_ELEMS = TJ * KS;
-    static constexpr int V_ELEMS = D * VS;
+    static constexpr int V_ELEMS = TJ * VS;
     static constexpr int STAGE = K_ELEMS + V_ELEMS;
     static constexpr int KCH = TJ * D / 8;                  // 16-byte K chunks per tile
-    static constexpr int NDP = D / 2;                       // column pairs of V
     static constexpr int SS = D + 8;                        // slab row stride (bf16)
     static constexpr int OS = D + 4;                        // accumulator row stride (fp32)
     // LDS carve-up (bytes)
@@ -122,59 +121,32 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     const int total_steps = nrounds * nt;
 
     // ---- staging of one K/V tile: global -> registers -> LDS ----------------
-    // K: KCH 16-byte chunks, V: 8 four-row groups x NDP column pairs; one of each
-    // per thread when D = 128, the first half of the threads when D = 64.
-    const bool k_owner = tid < C::KCH;
-    const int k_row = tid / (D / 8), k_col = tid - k_row * (D / 8);
-    const bool v_owner = tid < 8 * C::NDP;
-    const int v_dp = tid % C::NDP, v_grp = tid / C::NDP;
-    const uint32_t k_off = (uint32_t)k_row * (uint32_t)p.k1.sn + k_col * 8;
-    const uint32_t v_off = (uint32_t)(v_grp * 4) * (uint32_t)p.v1.sn + 2 * v_dp;
-    const uint32_t v_sn = (uint32_t)p.v1.sn;
-    uint4 kreg = make_uint4(0u, 0u, 0u, 0u);
-    uint32_t vreg[4] = {0u, 0u, 0u, 0u};
+    // Both tiles are copied row-major in 16-byte chunks, one K and one V chunk per thread
+    // (the first half of the threads when D = 64).
+    const bool t_owner = tid < C::KCH;
+    const int t_row = tid / (D / 8), t_col = tid - t_row * (D / 8);
+    const uint32_t k_off = (uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8;
+    const uint32_t v_off = (uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8;
+    uint4 kreg = make_uint4(0u, 0u, 0u, 0u), vreg = make_uint4(0u, 0u, 0u, 0u);
     auto load_tile = [&](int jt) {
         const int j0 = jt * TJ;
+        if (!t_owner) return;
         if (__builtin_expect(j0 + TJ <= N, 1)) {
-            if (k_owner) kreg = *(const uint4*)(k1p + (int64_t)j0 * p.k1.sn + k_off);
-            if (v_owner) {
-                const uint16_t* vb = v1p + (int64_t)j0 * p.v1.sn + v_off;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) vreg[r] = *(const uint32_t*)(vb + r * v_sn);
-            }
+            kreg = *(const uint4*)(k1p + (int64_t)j0 * p.k1.sn + k_off);
+            vreg = *(const uint4*)(v1p + (int64_t)j0 * p.v1.sn + v_off);
         } else {
             // last tile of the sequence: clamp the rows (they are masked later)
-            if (k_owner) {
-                int j = j0 + k_row;
-                j = j < N ? j : N - 1;
-                kreg = *(const uint4*)(k1p + (int64_t)j * p.k1.sn + k_col * 8);
-            }
-            if (v_owner) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    int j = j0 + v_grp * 4 + r;
-                    j = j < N ? j : N - 1;
-                    vreg[r] = *(const uint32_t*)(v1p + (int64_t)j * p.v1.sn + 2 * v_dp);
-                }
-            }
+            int j = j0 + t_row;
+            j = j < N ? j : N - 1;
+            kreg = *(const uint4*)(k1p + (int64_t)j * p.k1.sn + t_col * 8);
+            vreg = *(const uint4*)(v1p + (int64_t)j * p.v1.sn + t_col * 8);
         }
     };
-    auto store_tile = [&](int buf) {
-        uint16_t* Ks = smem + buf * C::STAGE;
-        uint16_t* Vt = Ks + C::K_ELEMS;
-        if (k_owner) *(uint4*)(Ks + k_row * C::KS + k_col * 8) = kreg;
-        if (v_owner) {
-            // key j = 8g + 4hh + t of the tile sits at position (g/2)*16 + hh*8 + (g%2)*4 + t
-            const int g = v_grp >> 1, hh = v_grp & 1;
-            const int pos = (g >> 1) * 16 + hh * 8 + (g & 1) * 4;
-            uint2 lo, hi;
-            lo.x = (vreg[0] & 0xffffu) | (vreg[1] << 16);
-            lo.y = (vreg[2] & 0xffffu) | (vreg[3] << 16);
-            hi.x = (vreg[0] >> 16) | (vreg[1] & 0xffff0000u);
-            hi.y = (vreg[2] >> 16) | (vreg[3] & 0xffff0000u);
-            *(uint2*)(Vt + (2 * v_dp) * C::VS + pos) = lo;
-            *(uint2*)(Vt + (2 * v_dp + 1) * C::VS + pos) = hi;
-        }
+    auto store_tile = [&](int b) {
+        if (!t_owner) return;
+        uint16_t* Ks = smem + b * C::STAGE;
+        *(uint4*)(Ks + t_row * C::KS + t_col * 8) = kreg;
+        *(uint4*)(Ks + C::K_ELEMS + t_row * C::VS + t_col * 8) = vreg;
     };
 
     // ---- workgroup accumulators ------------------------------------------------
@@ -316,7 +288,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
-                        const bf16x8 va = *(const bf16x8*)(Vt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                        const bf16x8 va = lds_column_operand(Vt + dt * 32, C::VS, ks, lane);
                         racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, w[ks], racc[dt], 0, 0, 0);
                     }
             };
@@ -422,7 +394,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks)
-                            va[dt][ks] = *(const bf16x8*)(Vt_prev + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                            va[dt][ks] = lds_column_operand(Vt_prev + dt * 32, C::VS, ks, lane);
                     floatx16 sh = negm;
                     if (__builtin_expect(!tile_plain(s), 0)) sh = masked_c((jt_lo + s) * TJ);
                     bf16x8 pb[2];
@@ -438,7 +410,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks)
                             racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK + 2 * C::DT, 0);       // the LDS reads
+                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK + 4 * C::DT, 0);       // the LDS reads
 #pragma unroll
                     for (int x = 0; x < C::DK; ++x) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
