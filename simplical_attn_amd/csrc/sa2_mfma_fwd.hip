@@ -396,7 +396,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                         for (int ks = 0; ks < 2; ++ks)
                             va[dt][ks] = lds_column_operand(Vt_prev + dt * 32, C::VS, ks, lane);
                     floatx16 sh = negm;
-                    if (__builtin_expect(!tile_plain(s), 0)) sh = masked_c((jt_lo + s) * TJ);
+                    if (__builtin_expect(!tile_plain(s), 0)) {
+                        asm volatile("" ::: "memory");      // keep the mask arithmetic out of the common path
+                        sh = masked_c((jt_lo + s) * TJ);
+                    }
                     bf16x8 pb[2];
                     float rs;
 #pragma unroll
