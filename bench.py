@@ -112,6 +112,9 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=2560)
+    ap.add_argument("--counters-only", action="store_true",
+                    help="for rocprofv3 --pmc runs: one 1 GiB device copy (the counter calibration), then two "
+                         "forward and two backward calls of the workload; prints no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (heads are independent and would "
@@ -135,6 +138,17 @@ def main():
     E = B * N * H * D
     fwd_bytes = 6 * E * 2 + 4 * B * H * N                  # read q,k1,k2,v1,v2; write O, LSE
     bwd_bytes = 12 * E * 2 + 12 * B * H * N                # read 5 inputs, O, dO; write 5 grads; LSE, D
+
+    if args.counters_only:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)                                   # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        for _ in range(2):
+            out, lse = sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2)
+            sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2)
+        torch.cuda.synchronize()
+        return
 
     leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
     attn = sa.TwoSimplicialAttention(D, w1, w2)

@@ -106,6 +106,29 @@ def test_extreme_and_zero_inputs():
     assert torch.allclose(lse[0, 0].cpu(), want.float(), rtol=1e-5)
 
 
+def test_repair_pass_when_logits_outgrow_the_first_reference_point():
+    """The fast kernel fixes a unit's softmax reference at its first tile; logits that
+    later grow by hundreds of octaves overflow its weights, the block is marked and the
+    repair kernel redoes it with a moving reference.  The result must still match."""
+    B, N, H, D, w1, w2 = 1, 160, 2, 64, 100, 5
+    q = torch.full((B, N, H, D), 0.5)
+    k2 = torch.full((B, N, H, D), 0.5)
+    ramp = torch.zeros(N)
+    ramp[40:] = 200.0                  # logit 0 on the first keys, 200 (288 octaves) later
+    ramp[120:] = 900.0
+    k1 = ramp[None, :, None, None].expand(B, N, H, D).contiguous()
+    g = torch.Generator().manual_seed(0)
+    v1 = torch.randn(B, N, H, D, generator=g)
+    v2 = torch.randn(B, N, H, D, generator=g)
+    inp = [t.to(torch.bfloat16) for t in (q, k1, k2, v1, v2)]
+    scale = 1.0 / (D * 0.25)           # s[i,j,k] = ramp[j]
+    out, lse = fwd(inp, w1, w2, scale)
+    want, want_lse = oracle_rows(inp, w1, w2, None, scale)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert_close_rel(out, want, BF16_TOL, "out")
+    assert_close_rel(lse, want_lse, BF16_TOL, "lse")
+
+
 def test_deterministic():
     inp = make_inputs(2, 300, 2, 128, seed=42, dtype=torch.bfloat16, with_dout=False)
     a = fwd(inp, 100, 20)
