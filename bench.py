@@ -43,7 +43,10 @@ WORKLOADS = {
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    ("c4", "forward"): 547.4e6,      # 371.4 MB read + 176.0 MB written
+    ("c4", "backward"): 13280.8e6,   # rowdot + row + finalize + column kernels, reads + writes
+}
 
 
 def count_triples(B, N, H, w1, w2):
