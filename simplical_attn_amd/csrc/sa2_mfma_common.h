@@ -53,6 +53,33 @@ __device__ __forceinline__ bf16x8 lds_column_operand(const uint16_t* tile, int s
     return u.v;
 }
 
+// The same operand from LDS byte addresses.  lds_column_lane_offset() is the per-lane part
+// (bytes, for ks = 0, relative to the 32x32 sub-block); lds_column_operand_at() takes the sum of
+// the sub-block's LDS byte address and that lane part, so that inside a loop the address is one
+// add and everything else sits in the instructions' immediate offsets.
+__device__ __forceinline__ uint32_t lds_column_lane_offset(int stride, int lane) {
+    const int grp = lane >> 4, s = lane & 15;
+    return (uint32_t)(((4 * (grp >> 1) + (s >> 2)) * stride + 16 * (grp & 1) + 4 * (s & 3)) * 2);
+}
+template <int STRIDE>
+__device__ __forceinline__ bf16x8 lds_column_operand_at(uint32_t addr, int ks) {
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef v4s __attribute__((address_space(3)))* lds_v4s;
+    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)(16 * ks * STRIDE * 2)));
+    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)((16 * ks + 8) * STRIDE * 2)));
+    union { v4s h[2]; bf16x8 v; } u;
+    u.h[0] = a;
+    u.h[1] = b;
+    return u.v;
+}
+// LDS byte address of a pointer into shared memory
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+__device__ __forceinline__ bf16x8 lds_read_bf16x8(uint32_t addr) {
+    return *(const bf16x8 __attribute__((address_space(3)))*)(uintptr_t)addr;
+}
+
 // acc *= alpha for an MFMA accumulator that lives in AGPRs, without asking the
 // register allocator for a VGPR copy of the tuple (it would place that copy on
 // the hot path).  Used only on the rare rescale path; the s_nop before the

@@ -125,28 +125,33 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     // (the first half of the threads when D = 64).
     const bool t_owner = tid < C::KCH;
     const int t_row = tid / (D / 8), t_col = tid - t_row * (D / 8);
-    const uint32_t k_off = (uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8;
-    const uint32_t v_off = (uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8;
+    // byte offsets of this thread's chunk from the first row of a tile; the tile's own
+    // offset is uniform, so a load is one instruction on a scalar base
+    const uint32_t k_off = ((uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8) * 2u;
+    const uint32_t v_off = ((uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8) * 2u;
+    uint32_t* st_dst = (uint32_t*)(smem + t_row * C::KS + t_col * 8);          // K chunk in stage 0
+    constexpr int V_SHIFT = C::K_ELEMS + 0;                                     // V tile follows the K tile
     uint4 kreg = make_uint4(0u, 0u, 0u, 0u), vreg = make_uint4(0u, 0u, 0u, 0u);
     auto load_tile = [&](int jt) {
         const int j0 = jt * TJ;
         if (!t_owner) return;
-        if (__builtin_expect(j0 + TJ <= N, 1)) {
-            kreg = *(const uint4*)(k1p + (int64_t)j0 * p.k1.sn + k_off);
-            vreg = *(const uint4*)(v1p + (int64_t)j0 * p.v1.sn + v_off);
-        } else {
+        uint32_t ko = k_off, vo = v_off;
+        if (__builtin_expect(j0 + TJ > N, 0)) {
             // last tile of the sequence: clamp the rows (they are masked later)
-            int j = j0 + t_row;
-            j = j < N ? j : N - 1;
-            kreg = *(const uint4*)(k1p + (int64_t)j * p.k1.sn + t_col * 8);
-            vreg = *(const uint4*)(v1p + (int64_t)j * p.v1.sn + t_col * 8);
+            const int r = t_row < N - 1 - j0 ? t_row : N - 1 - j0;
+            ko = ((uint32_t)r * (uint32_t)p.k1.sn + t_col * 8) * 2u;
+            vo = ((uint32_t)r * (uint32_t)p.v1.sn + t_col * 8) * 2u;
         }
+        const char* kb = (const char*)(k1p + (int64_t)j0 * p.k1.sn);
+        const char* vb = (const char*)(v1p + (int64_t)j0 * p.v1.sn);
+        kreg = *(const uint4*)(kb + ko);
+        vreg = *(const uint4*)(vb + vo);
     };
     auto store_tile = [&](int b) {
         if (!t_owner) return;
-        uint16_t* Ks = smem + b * C::STAGE;
-        *(uint4*)(Ks + t_row * C::KS + t_col * 8) = kreg;
-        *(uint4*)(Ks + C::K_ELEMS + t_row * C::VS + t_col * 8) = vreg;
+        uint16_t* Ks = (uint16_t*)st_dst + b * C::STAGE;
+        *(uint4*)Ks = kreg;
+        *(uint4*)(Ks + V_SHIFT + t_row * (C::VS - C::KS)) = vreg;
     };
 
     // ---- workgroup accumulators ------------------------------------------------
@@ -190,10 +195,16 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     };
 
     const float qscale = p.scale * LOG2E;
+    // LDS byte addresses: the stage ring, this lane's part of a K operand read (row ln, k-slots of
+    // its half) and of a transposed V operand read
+    const uint32_t smem_addr = lds_address(smem);
+    const uint32_t k_lane = (uint32_t)(ln * C::KS + hf * 8) * 2u;
+    const uint32_t v_lane = lds_column_lane_offset(C::VS, lane);
 
     load_tile(jt_lo);
     store_tile(0);
     if (total_steps > 1) load_tile(jt_lo + (1 % nt));
+    int next_tile = 2 % nt;                                     // tile index (from jt_lo) of step g + 2
     __syncthreads();
 
     // Tiles [s_lo, s_hi] need no mask: every key of the tile is inside the K window of
@@ -207,7 +218,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         // end of a tile step: next tile to LDS, the one after to registers, barrier
         const int nb = buf + 1 == C::NSTAGE ? 0 : buf + 1;
         if (g + 1 < total_steps) store_tile(nb);
-        if (g + 2 < total_steps) load_tile(jt_lo + (g + 2) % nt);
+        if (g + 2 < total_steps) load_tile(jt_lo + next_tile);
+        next_tile = next_tile + 1 == nt ? 0 : next_tile + 1;
         __syncthreads();
         buf = nb;
         ++g;
@@ -376,59 +388,73 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 // ---- two-stage software pipeline over the tiles: step t issues the logit MFMAs
                 // of tile t between the softmax instructions of tile t-1, then the value MFMAs
                 // of tile t-1; the shifted logits of tile t wait in registers for step t+1.
-                floatx16 sh_prev;
+                floatx16 sh_a, sh_b;
                 {
                     const floatx16 c0 = tile_plain(0) ? negm : masked_c(jt_lo * TJ);
-                    sh_prev = logit_mfmas(smem + buf * C::STAGE, c0);
+                    sh_a = logit_mfmas(smem + buf * C::STAGE, c0);
                 }
-                const uint16_t* Vt_prev = smem + buf * C::STAGE + C::K_ELEMS;
+                uint32_t vt_prev = smem_addr + (uint32_t)(buf * C::STAGE + C::K_ELEMS) * 2u + v_lane;
                 advance();
-                for (int s = 1; s < nt; ++s) {
-                    const uint16_t* Ks = smem + buf * C::STAGE;
-                    // all sixteen operand reads of the step go out first: the LDS latency is
-                    // paid once, not once per MFMA
-                    bf16x8 ka[C::DK], va[C::DT][2];
+                // One step: logits of tile s into `cur`, weights and value MFMAs of tile s-1 from `prev`.
+                auto step = [&](int s, const floatx16& prev, floatx16& cur) {
+                    const uint32_t ks_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u;
+                    bf16x8 ka[C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                        for (int ks = 0; ks < 2; ++ks)
-                            va[dt][ks] = lds_column_operand(Vt_prev + dt * 32, C::VS, ks, lane);
-                    floatx16 sh = negm;
-                    if (__builtin_expect(!tile_plain(s), 0)) {
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + k_lane + kk * 32);
+                    // the reference point (and, on the two window-edge tiles, the mask) is the
+                    // C operand of the first logit MFMA
+                    if (__builtin_expect(tile_plain(s), 1)) {
+                        cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], negm, 0, 0, 0);
+                    } else {
                         asm volatile("" ::: "memory");      // keep the mask arithmetic out of the common path
-                        sh = masked_c((jt_lo + s) * TJ);
+                        cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
                     }
                     bf16x8 pb[2];
                     float rs;
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk)
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sh, 0, 0, 0);
-                    weights(sh_prev, pb, rs);
+                    for (int kk = 1; kk < C::DK; ++kk)
+                        cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], cur, 0, 0, 0);
+                    weights(prev, pb, rs);
                     l += rs;
                     bad |= !(rs < OVERFLOW_LIMIT);
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                        for (int ks = 0; ks < 2; ++ks)
-                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK + 4 * C::DT, 0);       // the LDS reads
+                        for (int ks = 0; ks < 2; ++ks) {
+                            const bf16x8 va = lds_column_operand_at<C::VS>(vt_prev + dt * 64, ks);
+                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[ks], racc[dt], 0, 0, 0);
+                        }
 #pragma unroll
-                    for (int x = 0; x < C::DK; ++x) {
+                    for (int x = 1; x < C::DK; ++x) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x402, 48 / C::DK, 0);      // a slice of VALU / exp
+                        __builtin_amdgcn_sched_group_barrier(0x402, 5, 0);               // a slice of VALU / exp
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);               // two V operand reads
                     }
-                    sh_prev = sh;
-                    Vt_prev = Ks + C::K_ELEMS;
+                    vt_prev = ks_addr + (uint32_t)C::K_ELEMS * 2u + v_lane;
                     advance();
+                };
+                int s = 1;
+                for (; s + 1 < nt; s += 2) {
+                    step(s, sh_a, sh_b);
+                    step(s + 1, sh_b, sh_a);
                 }
                 bf16x8 pb[2];
                 float rs;
-                weights(sh_prev, pb, rs);
+                if (s < nt) {
+                    step(s, sh_a, sh_b);
+                    weights(sh_b, pb, rs);
+                } else {
+                    weights(sh_a, pb, rs);
+                }
                 l += rs;
                 bad |= !(rs < OVERFLOW_LIMIT);
-                value_mfmas(Vt_prev, pb);
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const bf16x8 va = lds_column_operand_at<C::VS>(vt_prev + dt * 64, ks);
+                        racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[ks], racc[dt], 0, 0, 0);
+                    }
             }
         }
 
