@@ -34,6 +34,13 @@ namespace sa2 {
 namespace {
 
 constexpr int FW = 8;                 // wavefronts per workgroup
+
+// The value of x behind a barrier the optimiser cannot see through: what is derived from it
+// is computed where it is used instead of being kept in a register across the tile sweep.
+__device__ __forceinline__ int recompute_here(int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
 constexpr int FT = FW * 64;           // threads per workgroup
 
 template <int D>
@@ -157,10 +164,16 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     // ---- workgroup accumulators ------------------------------------------------
     // thread -> (query aq, ACN columns from ac) of the fp32 accumulator in LDS
     constexpr int ACN = D / 16;                    // columns per thread (8 or 4)
-    const int aq = tid >> 4, ac = (tid & 15) * ACN;
+    {
+        const int aq = tid >> 4, ac = (tid & 15) * ACN;
 #pragma unroll
-    for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = 0.f;
-    float Mrun = -INFINITY, Lrun = 0.f;            // per query (lane), replicated in every wavefront
+        for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = 0.f;
+    }
+    // running maximum and sum of every query: fin_m / fin_l in LDS, read and updated at the merges
+    if (tid < BQ) {
+        fin_m[tid] = -INFINITY;
+        fin_l[tid] = 0.f;
+    }
     bool bad = false;
 
     // ---- q rows of the block and the K'/V' rows its deltas reach, once, to LDS ----
@@ -230,7 +243,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         const bool ok = delta < n_units;
         // The unit starts from the query's running reference point (finite from the second
         // round on), so only the first round has to look for maxima.
-        float m = ok ? Mrun : -INFINITY, l = 0.f;
+        float m = ok ? fin_m[ln] : -INFINITY, l = 0.f;
         floatx16 racc[C::DT];
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
@@ -409,6 +422,11 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                         asm volatile("" ::: "memory");      // keep the mask arithmetic out of the common path
                         cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
                     }
+                    bf16x8 va[C::DT][2];
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks) va[dt][ks] = lds_column_operand_at<C::VS>(vt_prev + dt * 64, ks);
                     bf16x8 pb[2];
                     float rs;
 #pragma unroll
@@ -421,8 +439,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) {
-                            const bf16x8 va = lds_column_operand_at<C::VS>(vt_prev + dt * 64, ks);
-                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[ks], racc[dt], 0, 0, 0);
+                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
                         }
 #pragma unroll
                     for (int x = 1; x < C::DK; ++x) {
@@ -459,29 +476,39 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         }
 
         // ---- fold the round's units into the workgroup accumulator --------------
+        // (lane coordinates are derived again here so that they do not occupy registers
+        // during the sweep)
+        const int tid_m = recompute_here(threadIdx.x);
+        const int ln_m = tid_m & 31, hf_m = (tid_m >> 5) & 1;
+        const int aq = tid_m >> 4, ac = (tid_m & 15) * ACN;
         const float lt = l + other_half(l);
-        if (hf == 0) {
-            xch_m[wave * BQ + ln] = m;
-            xch_l[wave * BQ + ln] = lt;
+        if (hf_m == 0) {
+            xch_m[wave * BQ + ln_m] = m;
+            xch_l[wave * BQ + ln_m] = lt;
         }
         __syncthreads();
+        const float Mrun = fin_m[ln_m], Lrun = fin_l[ln_m];
         float Mn = Mrun;
 #pragma unroll
-        for (int w = 0; w < FW; ++w) Mn = fmaxf(Mn, xch_m[w * BQ + ln]);
+        for (int w = 0; w < FW; ++w) Mn = fmaxf(Mn, xch_m[w * BQ + ln_m]);
         const float Muse = (Mn == -INFINITY) ? 0.f : Mn;
         const float a = fast_exp2(Mrun - Muse);
         float Ln = Lrun * a;
 #pragma unroll
-        for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln] * fast_exp2(xch_m[w * BQ + ln] - Muse);
-        Mrun = Mn;
-        Lrun = Ln;
-        if (wave == 0 && hf == 0) xch_a[ln] = a;
+        for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln_m] * fast_exp2(xch_m[w * BQ + ln_m] - Muse);
+        if (wave == 0 && hf_m == 0) xch_a[ln_m] = a;
         // Every wavefront writes its contribution c * (v2 + bias) * R as bf16 into its own
         // slab: four slabs have their own LDS, the other four use the two stage buffers
         // that hold no live tile between rounds.  Then every thread adds its slice of the
         // eight slabs in wavefront order.
         const float cw = ok ? fast_exp2(m - Muse) : 0.f;
-        const uint16_t* vrow = v2src + (int64_t)(ok ? side_row(delta) : 0) * v2stride + 4 * hf;
+        int vr;
+        if (side_kv) vr = ln_m + w2 - delta;
+        else {
+            const int iq = i0 + ln_m < N ? i0 + ln_m : N - 1;
+            vr = iq - delta > 0 ? iq - delta : 0;
+        }
+        const uint16_t* vrow = v2src + (int64_t)(ok ? vr : 0) * v2stride + 4 * hf_m;
         auto slab_of = [&](int w) -> uint16_t* {
             if (w < 4) return slabs + w * (BQ * C::SS);
             int fb = buf + 1 + ((w - 4) >> 1);                 // the two stage buffers other than buf
@@ -489,7 +516,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
             return smem + fb * C::STAGE + ((w - 4) & 1) * (BQ * C::SS);
         };
         {
-            uint16_t* srow = slab_of(wave) + ln * C::SS + 4 * hf;
+            uint16_t* srow = slab_of(wave) + ln_m * C::SS + 4 * hf_m;
 #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -504,6 +531,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 }
         }
         __syncthreads();
+        if (wave == 0 && hf_m == 0) {
+            fin_m[ln_m] = Mn;
+            fin_l[ln_m] = Ln;
+        }
         {
             const float ar = xch_a[aq];
             float acc[ACN];
@@ -530,11 +561,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
 
     // ---- normalise and store ------------------------------------------------------
     const bool any_bad = !SAFE && __syncthreads_or(bad ? 1 : 0);
-    if (wave == 0 && hf == 0) {
-        fin_m[ln] = Mrun;
-        fin_l[ln] = Lrun;
-    }
-    __syncthreads();
+    const int tid_f = recompute_here(threadIdx.x);
+    const int aq = tid_f >> 4, ac = (tid_f & 15) * ACN;
     const int io = i0 + aq;
     if (io < N) {
         const float Ms = fin_m[aq], L = fin_l[aq];
@@ -545,7 +573,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         for (int c = 0; c < ACN; ++c) o.h[c] = (__bf16)(oacc[aq * C::OS + ac + c] * inv);
         if (ACN == 8) *(uint4*)orow = o.u4;
         else *(uint2*)orow = o.u2;
-        if ((tid & 15) == 0) {
+        if ((tid_f & 15) == 0) {
             float lse;
             if (Ms > LOG2_EPS) lse = LN2 * (Ms + __log2f(L + 1e-8f * fast_exp2(-Ms)));
             else lse = LN_EPS + log1pf(L * fast_exp2(Ms - LOG2_EPS));
