@@ -619,6 +619,7 @@ bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
 
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
     (void)w1;
+    if (kp_fits(D, w2)) return kp_scratch_bytes(B, N, H, D, w2);
     const size_t one = (expanded_ws_bytes(B, N, H, D, w2) + 255) / 256 * 256;
     return 2 * one;
 }
@@ -627,7 +628,8 @@ int launch_mfma_bwd(const Problem& p, hipStream_t st) {
     int rc = launch_rowdot(p.out, p.dout, p.dsum, p.B, p.N, p.H, p.D, SA2_BF16, st);
     if (rc != SA2_OK) return rc;
     if (p.dq.p || p.dk2.p || p.dv2.p) {
-        rc = p.D == 128 ? launch_row_part<128>(p, st) : launch_row_part<64>(p, st);
+        if (kp_fits(p.D, p.w2)) rc = launch_mfma_bwd_kp(p, st);
+        else rc = p.D == 128 ? launch_row_part<128>(p, st) : launch_row_part<64>(p, st);
         if (rc != SA2_OK) return rc;
     }
     if (p.dk1.p || p.dv1.p) {

@@ -1,0 +1,586 @@
+// bf16 MFMA backward for gfx950, the K'-side kernel: dQ, dK' and dV'.
+//
+// Expanded rows r = (i, k), k = i - delta in the K' window of i.  A workgroup owns 32
+// consecutive K' rows k0..k0+31 and every delta: unit delta is the 32 rows
+// (i = k + delta, k).  With P = exp2(S - LSE*log2e) and dS = P * (dO~.v1 - D_i):
+//
+//   R[r,:] = sum_j P[r,j]  v1[j,:]        dV'[k] = sum_delta R[(k+delta,k)] * dO[k+delta]
+//   G[r,:] = sum_j dS[r,j] k1[j,:]        dK'[k] = scale * sum_delta G[(k+delta,k)] * q[k+delta]
+//                                         dQ[i]  = scale * sum_delta G[(i,i-delta)] * k2~[i-delta]
+//
+// dK' and dV' are aligned with the unit's rows, so they accumulate in registers over the
+// deltas a wavefront handles; dQ is shifted by delta and goes through an fp32 accumulator
+// in LDS (rows k0 .. k0+31+w2), written once per workgroup as a partial that a small
+// kernel adds up (a query gets partials from at most 2 + w2/32 workgroups, summed in a
+// fixed order: bitwise reproducible).
+//
+// Eight wavefronts, two per SIMD, form four pairs that each hold one unit per round and
+// sweep the K1/V1 window in 32-key tiles staged through a three-deep LDS ring:
+//   the "P" wavefront computes S^T = K1.Q~^T, P = exp2(S - LSE), hands P (bf16) to its
+//       partner through LDS and accumulates R^T += V1^T.P^T;
+//   the "dS" wavefront computes dP^T = V1.dO~^T and, one tile behind, dS = P*(dP - D) and
+//       G^T += K1^T.dS^T.
+// Every MFMA operand that streams from LDS is read once per 32x32x16 MFMA; transposed
+// operands come from the row-major tiles through ds_read_b64_tr_b16.
+#include "sa2_mfma_common.h"
+
+namespace sa2 {
+namespace {
+
+constexpr int KW = 8;                  // wavefronts per workgroup
+constexpr int KT = KW * 64;            // threads per workgroup
+constexpr int NPAIR = 4;
+
+__device__ __forceinline__ int kp_recompute_here(int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
+template <int D>
+struct KpCfg {
+    static constexpr int DK = D / 16;
+    static constexpr int DT = D / 32;
+    static constexpr int TS = D + 24;          // K/V tile row stride (bf16): full-rate row reads, good transpose reads
+    static constexpr int TILE = TJ * TS;
+    static constexpr int STAGE = 2 * TILE;     // K tile, then V tile
+    static constexpr int NSTAGE = 3;
+    static constexpr int KCH = TJ * D / 8;     // 16-byte chunks per tile
+    static constexpr int RS = D + 8;           // raw row / slab row stride (bf16)
+    static constexpr int AS = D + 4;           // fp32 accumulator row stride
+    static constexpr int PX_BYTES = NPAIR * 2 * 64 * 32;         // P hand-over, double buffered
+    static_assert(2 * BQ * RS <= STAGE, "two slabs must fit one stage buffer");
+    static constexpr size_t LDS_LIMIT = 160 * 1024;
+    static size_t main_bytes(int w2) {
+        const size_t rq = BQ + w2;
+        return (size_t)NSTAGE * STAGE * 2 + PX_BYTES + 2 * rq * RS * 2 + 2 * BQ * RS * 2 + 2 * ((rq + 3) / 4 * 4) * 4 + rq * AS * 4;
+    }
+    static size_t final_bytes() { return (size_t)KW * BQ * AS * 4; }
+    static size_t lds_bytes(int w2) { return main_bytes(w2) > final_bytes() ? main_bytes(w2) : final_bytes(); }
+    static bool fits(int w2) { return lds_bytes(w2) <= LDS_LIMIT; }
+};
+
+template <int D>
+__global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) {
+    using C = KpCfg<D>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int N = p.N, w1 = p.w1, w2 = p.w2;
+    const int RQ = BQ + w2;                                   // query rows this workgroup touches
+    uint16_t* smem = (uint16_t*)smem_raw;                     // stage ring
+    unsigned char* px = smem_raw + (size_t)C::NSTAGE * C::STAGE * 2;
+    uint16_t* q_s = (uint16_t*)(px + C::PX_BYTES);            // [RQ][RS] q rows k0 ..
+    uint16_t* do_s = q_s + RQ * C::RS;                        // [RQ][RS] dO rows
+    uint16_t* k2_s = do_s + RQ * C::RS;                       // [BQ][RS] K' rows k0 ..
+    uint16_t* v2_s = k2_s + BQ * C::RS;                       // [BQ][RS] V' rows
+    const int RQ4 = (RQ + 3) & ~3;
+    float* lse_s = (float*)(v2_s + BQ * C::RS);               // [RQ] LSE * log2(e)
+    float* dsum_s = lse_s + RQ4;                              // [RQ] D_i
+    float* dqacc = dsum_s + RQ4;                              // [RQ][AS]
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int role = wave >> 2, pr = wave & 3;                // role 0: P wavefront, 1: dS wavefront
+    const int lane = tid & 63, ln = lane & 31, hf = lane >> 5;
+
+    int pid = blockIdx.x;
+    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    const int bh = pid / nkb, kb = pid - bh * nkb;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int k0 = kb * BQ;
+    const int i_hi = (int)((int64_t)k0 + BQ - 1 + w2 < N - 1 ? k0 + BQ - 1 + w2 : N - 1);
+
+    const uint16_t* qp = (const uint16_t*)p.q.p + p.q.off(b, 0, h);
+    const uint16_t* k1p = (const uint16_t*)p.k1.p + p.k1.off(b, 0, h);
+    const uint16_t* k2p = (const uint16_t*)p.k2.p + p.k2.off(b, 0, h);
+    const uint16_t* v1p = (const uint16_t*)p.v1.p + p.v1.off(b, 0, h);
+    const uint16_t* v2p = (const uint16_t*)p.v2.p + p.v2.off(b, 0, h);
+    const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
+
+    const int jt_lo = (k0 - w1 > 0 ? k0 - w1 : 0) / TJ;
+    const int jt_hi = i_hi / TJ;
+    const int nt = jt_hi - jt_lo + 1;
+    const int n_units = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1;
+    const int nrounds = (n_units + NPAIR - 1) / NPAIR;
+    const int total_steps = nrounds * nt;
+    const bool want_dq = p.dq.p != nullptr;
+
+    // ---- staging of one K/V tile: global -> registers -> LDS (one K and one V chunk per thread)
+    const bool t_owner = tid < C::KCH;
+    const int t_row = tid / (D / 8), t_col = tid - t_row * (D / 8);
+    const uint32_t k_off = ((uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8) * 2u;
+    const uint32_t v_off = ((uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8) * 2u;
+    uint16_t* st_dst = smem + t_row * C::TS + t_col * 8;
+    uint4 kreg = make_uint4(0u, 0u, 0u, 0u), vreg = make_uint4(0u, 0u, 0u, 0u);
+    auto load_tile = [&](int jt) {
+        const int j0 = jt * TJ;
+        if (!t_owner) return;
+        uint32_t ko = k_off, vo = v_off;
+        if (__builtin_expect(j0 + TJ > N, 0)) {
+            const int r = t_row < N - 1 - j0 ? t_row : N - 1 - j0;        // clamp (masked later)
+            ko = ((uint32_t)r * (uint32_t)p.k1.sn + t_col * 8) * 2u;
+            vo = ((uint32_t)r * (uint32_t)p.v1.sn + t_col * 8) * 2u;
+        }
+        const char* kbp = (const char*)(k1p + (int64_t)j0 * p.k1.sn);
+        const char* vbp = (const char*)(v1p + (int64_t)j0 * p.v1.sn);
+        kreg = *(const uint4*)(kbp + ko);
+        vreg = *(const uint4*)(vbp + vo);
+    };
+    auto store_tile = [&](int sb) {
+        if (!t_owner) return;
+        uint16_t* Ks = st_dst + sb * C::STAGE;
+        *(uint4*)Ks = kreg;
+        *(uint4*)(Ks + C::TILE) = vreg;
+    };
+
+    // ---- raw rows, LSE, D and the dQ accumulator -------------------------------------
+    {
+        constexpr int CPR = D / 8;
+        for (int c = tid; c < RQ * CPR; c += KT) {
+            const int row = c / CPR, col = c - row * CPR;
+            int r = k0 + row;
+            r = r < N ? r : N - 1;
+            *(uint4*)(q_s + row * C::RS + col * 8) = *(const uint4*)(qp + (int64_t)r * p.q.sn + col * 8);
+            *(uint4*)(do_s + row * C::RS + col * 8) = *(const uint4*)(dop + (int64_t)r * p.dout.sn + col * 8);
+        }
+        for (int c = tid; c < BQ * CPR; c += KT) {
+            const int row = c / CPR, col = c - row * CPR;
+            int r = k0 + row;
+            r = r < N ? r : N - 1;
+            *(uint4*)(k2_s + row * C::RS + col * 8) = *(const uint4*)(k2p + (int64_t)r * p.k2.sn + col * 8);
+            *(uint4*)(v2_s + row * C::RS + col * 8) = *(const uint4*)(v2p + (int64_t)r * p.v2.sn + col * 8);
+        }
+        for (int c = tid; c < RQ; c += KT) {
+            int r = k0 + c;
+            r = r < N ? r : N - 1;
+            lse_s[c] = p.lse[(int64_t)bh * N + r] * LOG2E;
+            dsum_s[c] = p.dsum[(int64_t)bh * N + r];
+        }
+        for (int c = tid; c < RQ * C::AS; c += KT) dqacc[c] = 0.f;
+    }
+
+    const float qscale = p.scale * LOG2E;
+    const uint32_t smem_addr = lds_address(smem);
+    const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * 64 * 32 + lane * 32);
+    const uint32_t row_lane = (uint32_t)(ln * C::TS + hf * 8) * 2u;          // row operand: row ln, k-slots of this half
+    const uint32_t col_lane = lds_column_lane_offset(C::TS, lane);           // transposed operand
+
+    load_tile(jt_lo);
+    store_tile(0);
+    if (total_steps > 1) load_tile(jt_lo + (1 % nt));
+    int next_tile = 2 % nt;
+    __syncthreads();
+
+    int g = 0, buf = 0;
+    auto advance = [&]() {
+        const int nb = buf + 1 == C::NSTAGE ? 0 : buf + 1;
+        if (g + 1 < total_steps) store_tile(nb);
+        if (g + 2 < total_steps) load_tile(jt_lo + next_tile);
+        next_tile = next_tile + 1 == nt ? 0 : next_tile + 1;
+        __syncthreads();
+        buf = nb;
+        ++g;
+    };
+
+    // dV' (P wavefronts) or dK' (dS wavefronts) of this wavefront's deltas, rows k0+ln
+    floatx16 pacc[C::DT];
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) pacc[dt][v] = 0.f;
+
+    // slab of pair w for the dQ merge: the two stage buffers other than `buf`
+    auto slab_of = [&](int w) -> uint16_t* {
+        int fb = buf + 1 + (w >> 1);
+        fb = fb >= C::NSTAGE ? fb - C::NSTAGE : fb;
+        return smem + fb * C::STAGE + (w & 1) * (BQ * C::RS);
+    };
+    // add the round's four slabs (rows shifted by their delta) into the dQ accumulator
+    auto merge_dq = [&](int round) {
+        const int tid_m = kp_recompute_here(threadIdx.x);
+        constexpr int CH = D / 16;
+        for (int it = tid_m; it < RQ * CH; it += KT) {
+            const int row = it / CH, c0 = (it - row * CH) * 16;
+            float acc[16];
+#pragma unroll
+            for (int c = 0; c < 16; ++c) acc[c] = 0.f;
+#pragma unroll
+            for (int w = 0; w < NPAIR; ++w) {
+                const int dl = round * NPAIR + w;
+                const int kl = row - dl;
+                if (dl < n_units && kl >= 0 && kl < BQ) {
+                    const uint16_t* sp = slab_of(w) + kl * C::RS + c0;
+                    const uint4 x = *(const uint4*)sp, y = *(const uint4*)(sp + 8);
+                    acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
+                    acc[4] += bf16_lo(x.z); acc[5] += bf16_hi(x.z); acc[6] += bf16_lo(x.w); acc[7] += bf16_hi(x.w);
+                    acc[8] += bf16_lo(y.x); acc[9] += bf16_hi(y.x); acc[10] += bf16_lo(y.y); acc[11] += bf16_hi(y.y);
+                    acc[12] += bf16_lo(y.z); acc[13] += bf16_hi(y.z); acc[14] += bf16_lo(y.w); acc[15] += bf16_hi(y.w);
+                }
+            }
+            float* ap = dqacc + row * C::AS + c0;
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                float4 a = *(float4*)(ap + 4 * c4);
+                a.x += acc[4 * c4]; a.y += acc[4 * c4 + 1]; a.z += acc[4 * c4 + 2]; a.w += acc[4 * c4 + 3];
+                *(float4*)(ap + 4 * c4) = a;
+            }
+        }
+    };
+
+    if (role == 0) {
+        // =============================== P wavefronts ================================
+        for (int round = 0; round < nrounds; ++round) {
+            const int delta = round * NPAIR + pr;
+            const bool ok = delta < n_units;
+            const int i = k0 + ln + delta;
+            const bool row_ok = i < N;
+            const int i_min = k0 + delta;
+            const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
+            const bool rows_full = i_min + BQ - 1 < N;
+            const int sa = ok ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;     // first and last tile of the unit
+            const int sb = ok ? i_max / TJ - jt_lo : -1;
+            floatx16 racc[C::DT];
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) racc[dt][v] = 0.f;
+            bf16x8 qf[C::DK];
+            float lse2 = 0.f;
+            {
+                const uint16_t* qrow = q_s + (ln + delta) * C::RS + hf * 8;
+                const uint16_t* krow = k2_s + ln * C::RS + hf * 8;
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) {
+                    const uint4 qa = *(const uint4*)(qrow + kk * 16);
+                    const uint4 kx = *(const uint4*)(krow + kk * 16);
+                    const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
+                    const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w};
+                    bf16x8 r;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
+                        r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
+                    }
+                    qf[kk] = r;
+                }
+                if (ok) lse2 = lse_s[ln + delta];
+            }
+            for (int s = 0; s < nt; ++s) {
+                if (s >= sa && s <= sb) {
+                    const int j0 = (jt_lo + s) * TJ;
+                    const uint32_t ks_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u;
+                    bf16x8 ka[C::DK];
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + row_lane + kk * 32);
+                    floatx16 sh;
+                    const bool plain = rows_full && j0 + TJ - 1 <= i_min && j0 >= i_max - w1;
+                    if (__builtin_expect(plain, 1)) {
+                        floatx16 zero;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], zero, 0, 0, 0);
+                    } else {
+                        asm volatile("" ::: "memory");
+                        // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
+                        const int hi = i - j0 - 4 * hf, lo = hi - w1;
+                        floatx16 ct;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = 8 * (v >> 2) + (v & 3);
+                            ct[v] = (row_ok & (c <= hi) & (c >= lo)) ? 0.f : -INFINITY;
+                        }
+                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], ct, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int kk = 1; kk < C::DK; ++kk)
+                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sh, 0, 0, 0);
+                    bf16x8 pb[2];
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) pb[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t] - lse2);
+                    {
+                        typedef bf16x8 __attribute__((address_space(3)))* lds_b8;
+                        const uint32_t a = px_addr + (uint32_t)((g & 1) * 64 * 32);
+                        *(lds_b8)(uintptr_t)a = pb[0];
+                        *(lds_b8)(uintptr_t)(a + 16) = pb[1];
+                    }
+                    const uint32_t vt_addr = ks_addr + (uint32_t)C::TILE * 2u + col_lane;
+                    bf16x8 va[C::DT][2];
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks) va[dt][ks] = lds_column_operand_at<C::TS>(vt_addr + dt * 64, ks);
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks)
+                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
+                }
+                advance();
+            }
+            // dV'[k] += R[(k+delta, k)] * dO[k+delta]
+            if (ok) {
+                const uint16_t* drow = do_s + (ln + delta) * C::RS + 4 * hf;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = *(const uint2*)(drow + dt * 32 + 8 * g4);
+                        pacc[dt][4 * g4 + 0] += racc[dt][4 * g4 + 0] * bf16_lo(x.x);
+                        pacc[dt][4 * g4 + 1] += racc[dt][4 * g4 + 1] * bf16_hi(x.x);
+                        pacc[dt][4 * g4 + 2] += racc[dt][4 * g4 + 2] * bf16_lo(x.y);
+                        pacc[dt][4 * g4 + 3] += racc[dt][4 * g4 + 3] * bf16_hi(x.y);
+                    }
+            }
+            if (want_dq) {
+                __syncthreads();       // the dS wavefronts are done with the last tile
+                __syncthreads();       // slabs written
+                merge_dq(round);
+                __syncthreads();       // the stage buffers that served as slabs are free again
+            }
+        }
+    } else {
+        // =============================== dS wavefronts ===============================
+        for (int round = 0; round < nrounds; ++round) {
+            const int delta = round * NPAIR + pr;
+            const bool ok = delta < n_units;
+            const int i_min = k0 + delta;
+            const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
+            const int sa = ok ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;
+            const int sb = ok ? i_max / TJ - jt_lo : -1;
+            floatx16 gacc[C::DT];
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) gacc[dt][v] = 0.f;
+            bf16x8 dof[C::DK];
+            float dsum = 0.f;
+            {
+                const uint16_t* drow = do_s + (ln + delta) * C::RS + hf * 8;
+                const uint16_t* vrow = v2_s + ln * C::RS + hf * 8;
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) {
+                    const uint4 da = *(const uint4*)(drow + kk * 16);
+                    const uint4 vx = *(const uint4*)(vrow + kk * 16);
+                    const uint32_t dw[4] = {da.x, da.y, da.z, da.w};
+                    const uint32_t vw[4] = {vx.x, vx.y, vx.z, vx.w};
+                    bf16x8 r;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        r[2 * t] = (__bf16)(bf16_lo(dw[t]) * (bf16_lo(vw[t]) + p.v2_bias));
+                        r[2 * t + 1] = (__bf16)(bf16_hi(dw[t]) * (bf16_hi(vw[t]) + p.v2_bias));
+                    }
+                    dof[kk] = r;
+                }
+                if (ok) dsum = dsum_s[ln + delta];
+            }
+            floatx16 dp_prev;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dp_prev[v] = 0.f;
+            // dS of the tile handled in the previous step and its G MFMAs
+            auto consume = [&]() {
+                typedef const bf16x8 __attribute__((address_space(3)))* lds_b8;
+                const uint32_t a = px_addr + (uint32_t)(((g - 1) & 1) * 64 * 32);
+                const bf16x8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
+                const int pb = buf == 0 ? C::NSTAGE - 1 : buf - 1;
+                const uint32_t kt_addr = smem_addr + (uint32_t)(pb * C::STAGE) * 2u + col_lane;
+                bf16x8 kt[C::DT][2];
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) kt[dt][ks] = lds_column_operand_at<C::TS>(kt_addr + dt * 64, ks);
+                bf16x8 dsb[2];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    dsb[0][t] = (__bf16)((float)p0[t] * (dp_prev[t] - dsum));
+                    dsb[1][t] = (__bf16)((float)p1[t] * (dp_prev[8 + t] - dsum));
+                }
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+                        gacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt[dt][ks], dsb[ks], gacc[dt], 0, 0, 0);
+            };
+            for (int s = 0; s < nt; ++s) {
+                floatx16 dp;
+                const bool act = s >= sa && s <= sb;
+                if (act) {
+                    const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE + C::TILE) * 2u;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) dp[v] = 0.f;
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) {
+                        const bf16x8 va = lds_read_bf16x8(vs_addr + row_lane + kk * 32);
+                        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp, 0, 0, 0);
+                    }
+                }
+                if (s - 1 >= sa && s - 1 <= sb) consume();
+                if (act) dp_prev = dp;
+                advance();
+            }
+            if (nt - 1 >= sa && nt - 1 <= sb) consume();
+            // dK'[k] += G[(k+delta, k)] * q[k+delta]   (scale applied at the end)
+            if (ok) {
+                const uint16_t* qrow = q_s + (ln + delta) * C::RS + 4 * hf;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = *(const uint2*)(qrow + dt * 32 + 8 * g4);
+                        pacc[dt][4 * g4 + 0] += gacc[dt][4 * g4 + 0] * bf16_lo(x.x);
+                        pacc[dt][4 * g4 + 1] += gacc[dt][4 * g4 + 1] * bf16_hi(x.x);
+                        pacc[dt][4 * g4 + 2] += gacc[dt][4 * g4 + 2] * bf16_lo(x.y);
+                        pacc[dt][4 * g4 + 3] += gacc[dt][4 * g4 + 3] * bf16_hi(x.y);
+                    }
+            }
+            if (want_dq) {
+                __syncthreads();       // every dS wavefront is done with the last tile
+                if (ok) {
+                    // dQ contribution of the unit: scale * G * k2~, row ln of the slab is query k0+ln+delta
+                    uint16_t* srow = slab_of(pr) + ln * C::RS + 4 * hf;
+                    const uint16_t* krow = k2_s + ln * C::RS + 4 * hf;
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int g4 = 0; g4 < 4; ++g4) {
+                            const uint2 x = *(const uint2*)(krow + dt * 32 + 8 * g4);
+                            union { __bf16 h[4]; uint2 u; } o;
+                            o.h[0] = (__bf16)(p.scale * gacc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.k2_bias));
+                            o.h[1] = (__bf16)(p.scale * gacc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.k2_bias));
+                            o.h[2] = (__bf16)(p.scale * gacc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.k2_bias));
+                            o.h[3] = (__bf16)(p.scale * gacc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.k2_bias));
+                            *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
+                        }
+                }
+                __syncthreads();
+                merge_dq(round);
+                __syncthreads();
+            }
+        }
+    }
+
+    // ---- dQ partial of this workgroup ------------------------------------------------
+    const int tid_f = kp_recompute_here(threadIdx.x);
+    __syncthreads();
+    if (want_dq) {
+        constexpr int CH = D / 4;
+        float* dst = dq_part + ((int64_t)bh * nkb + kb) * RQ * D;
+        for (int it = tid_f; it < RQ * CH; it += KT) {
+            const int row = it / CH, c0 = (it - row * CH) * 4;
+            *(float4*)(dst + (int64_t)row * D + c0) = *(const float4*)(dqacc + row * C::AS + c0);
+        }
+    }
+    __syncthreads();
+    // ---- dK' and dV': add the four wavefronts of each role through LDS ----------------
+    {
+        float* region = (float*)smem_raw + (size_t)wave * BQ * C::AS;
+        const int ln_f = tid_f & 31, hf_f = (tid_f >> 5) & 1;
+        float* rrow = region + ln_f * C::AS + 4 * hf_f;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                float4 a;
+                a.x = pacc[dt][4 * g4 + 0]; a.y = pacc[dt][4 * g4 + 1];
+                a.z = pacc[dt][4 * g4 + 2]; a.w = pacc[dt][4 * g4 + 3];
+                *(float4*)(rrow + dt * 32 + 8 * g4) = a;
+            }
+    }
+    __syncthreads();
+    {
+        constexpr int CH = D / 8;
+        const float* base = (const float*)smem_raw;
+        for (int it = tid_f; it < 2 * BQ * CH; it += KT) {
+            const int which = it / (BQ * CH);                       // 0: dV' (P wavefronts), 1: dK'
+            const int rem = it - which * BQ * CH;
+            const int row = rem / CH, c0 = (rem - row * CH) * 8;
+            const int k = k0 + row;
+            const Tensor& t = which ? p.dk2 : p.dv2;
+            if (k >= N || !t.p) continue;
+            float acc[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[c] = 0.f;
+#pragma unroll
+            for (int w = 0; w < NPAIR; ++w) {
+                const float* rp = base + (size_t)(which * NPAIR + w) * BQ * C::AS + row * C::AS + c0;
+                const float4 a = *(const float4*)rp, c4 = *(const float4*)(rp + 4);
+                acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
+                acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
+            }
+            const float sc = which ? p.scale : 1.f;
+            union { __bf16 hh[8]; uint4 u; } o;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) o.hh[c] = (__bf16)(acc[c] * sc);
+            *(uint4*)((uint16_t*)t.p + t.off(b, k, h) + c0) = o.u;
+        }
+    }
+}
+
+// dQ[i] = sum of the partials of the K' blocks that reach query i, in block order.
+template <int D>
+__global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const float* __restrict__ dq_part, int nkb,
+                                                             int64_t items) {
+    constexpr int CH = D / 8;
+    const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (it >= items) return;
+    const int c0 = (int)(it % CH) * 8;
+    const int64_t row = it / CH;
+    const int N = p.N, RQ = BQ + p.w2;
+    const int i = (int)(row % N);
+    const int bh = (int)(row / N);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int kb_hi = i / BQ;
+    int kb_lo = (i - RQ + BQ) / BQ;              // smallest kb with i - 32*kb <= RQ-1
+    kb_lo = (i - RQ + 1 <= 0) ? 0 : kb_lo;
+    float acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] = 0.f;
+    for (int kb = kb_lo; kb <= kb_hi; ++kb) {
+        const float* src = dq_part + (((int64_t)bh * nkb + kb) * RQ + (i - kb * BQ)) * D + c0;
+        const float4 a = *(const float4*)src, c4 = *(const float4*)(src + 4);
+        acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
+        acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
+    }
+    union { __bf16 hh[8]; uint4 u; } o;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) o.hh[c] = (__bf16)acc[c];
+    *(uint4*)((uint16_t*)p.dq.p + p.dq.off(b, i, h) + c0) = o.u;
+}
+
+template <int D>
+int launch_kp(const Problem& p, hipStream_t st) {
+    using C = KpCfg<D>;
+    const int nkb = (p.N + BQ - 1) / BQ;
+    const int64_t total = (int64_t)nkb * p.B * p.H;
+    if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
+    if (p.dq.p && p.scratch_bytes < kp_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+    const size_t lds = C::lds_bytes(p.w2);
+    if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+        return SA2_ERR_LAUNCH_FAILED;
+    float* part = (float*)p.scratch;
+    hipLaunchKernelGGL(mfma_bwd_kp_kernel<D>, dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part);
+    if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    if (p.dq.p) {
+        const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
+        hipLaunchKernelGGL(mfma_bwd_dq_sum_kernel<D>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p, part,
+                           nkb, items);
+        if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    }
+    return SA2_OK;
+}
+
+}  // namespace
+
+bool kp_fits(int D, int w2) { return D == 128 ? KpCfg<128>::fits(w2) : (D == 64 ? KpCfg<64>::fits(w2) : false); }
+
+size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {
+    const size_t nkb = (size_t)(N + BQ - 1) / BQ;
+    return (size_t)B * H * nkb * (size_t)(BQ + w2) * D * sizeof(float);
+}
+
+int launch_mfma_bwd_kp(const Problem& p, hipStream_t st) {
+    return p.D == 128 ? launch_kp<128>(p, st) : launch_kp<64>(p, st);
+}
+
+}  // namespace sa2
