@@ -82,5 +82,8 @@ size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 bool kp_fits(int D, int w2);
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2);
 int launch_mfma_bwd_kp(const Problem& p, hipStream_t st);
+// K-side backward kernel (dK, dV) with paired wavefronts
+bool kv_fits(int D, int w2);
+int launch_mfma_bwd_kv(const Problem& p, hipStream_t st);
 
 }  // namespace sa2

@@ -633,7 +633,8 @@ int launch_mfma_bwd(const Problem& p, hipStream_t st) {
         if (rc != SA2_OK) return rc;
     }
     if (p.dk1.p || p.dv1.p) {
-        rc = p.D == 128 ? launch_col_part<128>(p, st) : launch_col_part<64>(p, st);
+        if (kv_fits(p.D, p.w2)) rc = launch_mfma_bwd_kv(p, st);
+        else rc = p.D == 128 ? launch_col_part<128>(p, st) : launch_col_part<64>(p, st);
     }
     return rc;
 }
