@@ -72,6 +72,56 @@ __device__ __forceinline__ bf16x8 lds_column_operand_at(uint32_t addr, int ks) {
     u.h[1] = b;
     return u.v;
 }
+// Tiles written by direct global->LDS loads keep groups of RPW rows together: within a group
+// the 16-byte chunk c of row q sits at byte (c * RPW + q) * 16, groups lie GROUP bytes apart.
+// Transposed MFMA operand out of such a tile (same lanes and k-slot order as
+// lds_column_operand): the lane part of the address, and the two reads of k-step ks of the
+// 32-column block whose byte address (block * 64 * RPW) is already in `addr`.
+template <int RPW, int GROUP>
+__device__ __forceinline__ uint32_t lds_group_column_lane_offset(int lane) {
+    const int grp = lane >> 4, s = lane & 15;
+    const int rr = 4 * (grp >> 1) + (s >> 2);            // row within the 8-row slice
+    const int cc = 16 * (grp & 1) + 4 * (s & 3);         // column within the 32-column block
+    return (uint32_t)((rr / RPW) * GROUP + ((cc / 8) * RPW + rr % RPW) * 16 + (cc % 8) * 2);
+}
+template <int RPW, int GROUP>
+__device__ __forceinline__ bf16x8 lds_group_column_operand(uint32_t addr, int ks) {
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef v4s __attribute__((address_space(3)))* lds_v4s;
+    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)((16 * ks / RPW) * GROUP)));
+    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)(((16 * ks + 8) / RPW) * GROUP)));
+    union { v4s h[2]; bf16x8 v; } u;
+    u.h[0] = a;
+    u.h[1] = b;
+    return u.v;
+}
+// The same operand read in two phases for loops that keep direct global->LDS loads in
+// flight: the compiler would wait for every outstanding vector-memory operation before a
+// transpose-read builtin, so the reads are issued as opaque instructions and the wait for
+// their results is placed by hand (lds_settle) before the first use.
+typedef short lds_half_operand __attribute__((ext_vector_type(4)));
+template <int OFF_A, int OFF_B>
+__device__ __forceinline__ void lds_tr_issue(uint32_t addr, lds_half_operand& a, lds_half_operand& b) {
+    asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                 : "=&v"(a), "=&v"(b)
+                 : "v"(addr), "n"(OFF_A), "n"(OFF_B));
+}
+// all LDS reads issued so far have returned; the operands named here are only used afterwards
+__device__ __forceinline__ void lds_settle(lds_half_operand (&x)[16]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]),
+                   "+v"(x[8]), "+v"(x[9]), "+v"(x[10]), "+v"(x[11]), "+v"(x[12]), "+v"(x[13]), "+v"(x[14]), "+v"(x[15]));
+}
+__device__ __forceinline__ void lds_settle(lds_half_operand (&x)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]));
+}
+__device__ __forceinline__ bf16x8 lds_join(const lds_half_operand& a, const lds_half_operand& b) {
+    union { lds_half_operand h[2]; bf16x8 v; } u;
+    u.h[0] = a;
+    u.h[1] = b;
+    return u.v;
+}
 // LDS byte address of a pointer into shared memory
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;

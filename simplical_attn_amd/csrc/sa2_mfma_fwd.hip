@@ -47,18 +47,22 @@ template <int D>
 struct Cfg {
     static constexpr int DK = D / 16;          // k-steps of the logit contraction
     static constexpr int DT = D / 32;          // 32-column tiles of the value contraction
-    static constexpr int KS = D + 8;           // K tile row stride in LDS (bf16), +16 B against bank conflicts
-    static constexpr int VS = D + 16;          // V tile row stride in LDS (bf16), +32 B: conflict-free transpose reads
-    static constexpr int K_ELEMS = TJ * KS;
-    static constexpr int V_ELEMS = TJ * VS;
-    static constexpr int STAGE = K_ELEMS + V_ELEMS;
-    static constexpr int KCH = TJ * D / 8;                  // 16-byte K chunks per tile
+    static constexpr int KS = D + 8;           // row stride of the q / K' / V' copies in LDS (bf16)
+    // A K or V tile in LDS is written by direct global->LDS loads: one wavefront instruction
+    // fills a group of RPW rows (1 KB), lane L putting the 16-byte chunk L / RPW of row
+    // L % RPW at byte 16 * L.  Groups lie GROUP bytes apart.  Row operand reads and
+    // transposed operand reads are both bank-conflict free in this layout.
+    static constexpr int RPW = 512 / D;                     // rows per group: 4 (D = 128) or 8 (D = 64)
+    static constexpr int GROUP = 1024 + 16 * RPW;           // bytes
+    static constexpr int NGROUP = TJ / RPW;
+    static constexpr int TILE_BYTES = NGROUP * GROUP;
+    static constexpr int STAGE = TILE_BYTES;                // bf16 elements of one stage = K tile + V tile
     static constexpr int SS = D + 8;                        // slab row stride (bf16)
     static constexpr int OS = D + 4;                        // accumulator row stride (fp32)
     // LDS carve-up (bytes)
-    static constexpr int NSTAGE = 3;
+    static constexpr int NSTAGE = 4;
     static constexpr size_t STAGE_BYTES = (size_t)NSTAGE * STAGE * 2;
-    static constexpr size_t SLAB_BYTES = (size_t)4 * BQ * SS * 2;          // four slabs; four more live in idle stage buffers
+    static constexpr size_t SLAB_BYTES = (size_t)2 * BQ * SS * 2;          // two slabs; six more live in idle stage buffers
     static_assert(2 * BQ * SS <= STAGE, "two slabs must fit one stage buffer");
     static constexpr size_t OACC_BYTES = (size_t)BQ * OS * 4;
     static constexpr size_t XCH_BYTES = (size_t)(2 * FW * BQ + 3 * BQ) * 4;
@@ -127,38 +131,35 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     const int nrounds = (n_units + FW - 1) / FW;
     const int total_steps = nrounds * nt;
 
-    // ---- staging of one K/V tile: global -> registers -> LDS ----------------
-    // Both tiles are copied row-major in 16-byte chunks, one K and one V chunk per thread
-    // (the first half of the threads when D = 64).
-    const bool t_owner = tid < C::KCH;
-    const int t_row = tid / (D / 8), t_col = tid - t_row * (D / 8);
-    // byte offsets of this thread's chunk from the first row of a tile; the tile's own
-    // offset is uniform, so a load is one instruction on a scalar base
+    // ---- staging of one K/V tile: direct global -> LDS loads ------------------------
+    // Wavefront w fills group w of the K tile and of the V tile (the first NGROUP wavefronts
+    // when D = 64).  Tiles are requested strictly in sweep order into consecutive ring stages.
+    const bool t_owner = wave < C::NGROUP;
+    const int t_row = wave * C::RPW + (lane % C::RPW), t_col = lane / C::RPW;
     const uint32_t k_off = ((uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8) * 2u;
     const uint32_t v_off = ((uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8) * 2u;
-    uint32_t* st_dst = (uint32_t*)(smem + t_row * C::KS + t_col * 8);          // K chunk in stage 0
-    constexpr int V_SHIFT = C::K_ELEMS + 0;                                     // V tile follows the K tile
-    uint4 kreg = make_uint4(0u, 0u, 0u, 0u), vreg = make_uint4(0u, 0u, 0u, 0u);
-    auto load_tile = [&](int jt) {
-        const int j0 = jt * TJ;
-        if (!t_owner) return;
-        uint32_t ko = k_off, vo = v_off;
-        if (__builtin_expect(j0 + TJ > N, 0)) {
-            // last tile of the sequence: clamp the rows (they are masked later)
-            const int r = t_row < N - 1 - j0 ? t_row : N - 1 - j0;
-            ko = ((uint32_t)r * (uint32_t)p.k1.sn + t_col * 8) * 2u;
-            vo = ((uint32_t)r * (uint32_t)p.v1.sn + t_col * 8) * 2u;
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    typedef const __attribute__((address_space(1))) void* glb_ptr;
+    int dma_tile = 0, dma_stage = 0, dma_count = 0;             // next tile (from jt_lo), its stage, tiles requested
+    auto dma_next = [&]() {
+        const int j0 = (jt_lo + dma_tile) * TJ;
+        if (t_owner) {
+            uint32_t ko = k_off, vo = v_off;
+            if (__builtin_expect(j0 + TJ > N, 0)) {
+                // last tile of the sequence: clamp the rows (they are masked later)
+                const int r = t_row < N - 1 - j0 ? t_row : N - 1 - j0;
+                ko = ((uint32_t)r * (uint32_t)p.k1.sn + t_col * 8) * 2u;
+                vo = ((uint32_t)r * (uint32_t)p.v1.sn + t_col * 8) * 2u;
+            }
+            const char* kb = (const char*)(k1p + (int64_t)j0 * p.k1.sn);
+            const char* vb = (const char*)(v1p + (int64_t)j0 * p.v1.sn);
+            unsigned char* dst = smem_raw + (size_t)dma_stage * (C::STAGE * 2) + wave * C::GROUP;
+            __builtin_amdgcn_global_load_lds((glb_ptr)(kb + ko), (lds_ptr)dst, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_ptr)(vb + vo), (lds_ptr)(dst + C::TILE_BYTES), 16, 0, 0);
         }
-        const char* kb = (const char*)(k1p + (int64_t)j0 * p.k1.sn);
-        const char* vb = (const char*)(v1p + (int64_t)j0 * p.v1.sn);
-        kreg = *(const uint4*)(kb + ko);
-        vreg = *(const uint4*)(vb + vo);
-    };
-    auto store_tile = [&](int b) {
-        if (!t_owner) return;
-        uint16_t* Ks = (uint16_t*)st_dst + b * C::STAGE;
-        *(uint4*)Ks = kreg;
-        *(uint4*)(Ks + V_SHIFT + t_row * (C::VS - C::KS)) = vreg;
+        dma_tile = dma_tile + 1 == nt ? 0 : dma_tile + 1;
+        dma_stage = (dma_stage + 1) & (C::NSTAGE - 1);
+        ++dma_count;
     };
 
     // ---- workgroup accumulators ------------------------------------------------
@@ -211,13 +212,13 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     // LDS byte addresses: the stage ring, this lane's part of a K operand read (row ln, k-slots of
     // its half) and of a transposed V operand read
     const uint32_t smem_addr = lds_address(smem);
-    const uint32_t k_lane = (uint32_t)(ln * C::KS + hf * 8) * 2u;
-    const uint32_t v_lane = lds_column_lane_offset(C::VS, lane);
+    const uint32_t k_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);
+    const uint32_t v_lane = lds_group_column_lane_offset<C::RPW, C::GROUP>(lane);
 
-    load_tile(jt_lo);
-    store_tile(0);
-    if (total_steps > 1) load_tile(jt_lo + (1 % nt));
-    int next_tile = 2 % nt;                                     // tile index (from jt_lo) of step g + 2
+    dma_next();
+    if (total_steps > 1) dma_next();
+    if (total_steps > 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     // Tiles [s_lo, s_hi] need no mask: every key of the tile is inside the K window of
@@ -226,15 +227,21 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     s_lo = (i0 + BQ - 1 - w1 <= jt_lo * TJ) ? 0 : s_lo;
     const int s_hi = (i0 + 1) / TJ - 1 - jt_lo;                 // last tile with j0+31 <= i0
 
+    // Step g of the sweep works on ring stage g % NSTAGE.  At its start the tile of step g+2 is
+    // requested (the stage it goes to was last read in step g-1); at its end the tile of step
+    // g+1 must have landed.  The last step of a round requests nothing, so that three stages
+    // are free for the merge; the first step of the next round catches up.
     int g = 0, buf = 0;                                         // buf = g % NSTAGE
+    bool requested = false;
+    auto begin_step = [&](int s) {
+        if (s == 0 && g > 0 && dma_count < total_steps) dma_next();
+        requested = s + 1 < nt && dma_count < total_steps;
+        if (requested) dma_next();
+    };
     auto advance = [&]() {
-        // end of a tile step: next tile to LDS, the one after to registers, barrier
-        const int nb = buf + 1 == C::NSTAGE ? 0 : buf + 1;
-        if (g + 1 < total_steps) store_tile(nb);
-        if (g + 2 < total_steps) load_tile(jt_lo + next_tile);
-        next_tile = next_tile + 1 == nt ? 0 : next_tile + 1;
-        __syncthreads();
-        buf = nb;
+        if (requested) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        buf = (buf + 1) & (C::NSTAGE - 1);
         ++g;
     };
 
@@ -252,7 +259,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
 
         if (!ok) {
             // no unit for this wavefront in this round: keep the staging pipeline moving
-            for (int s = 0; s < nt; ++s) advance();
+            for (int s = 0; s < nt; ++s) {
+                begin_step(s);
+                advance();
+            }
         } else {
             // ---- new unit: Q~ operand, fresh softmax state ----------------------
             bf16x8 qf[C::DK];
@@ -300,20 +310,38 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 }
                 rsum = r;
             };
-            auto logit_mfmas = [&](const uint16_t* Ks, floatx16 c) -> floatx16 {
+            constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;      // operand strides of a k-step / a 32-column block
+            auto stage_addr = [&](int st) { return smem_addr + (uint32_t)st * (uint32_t)(C::STAGE * 2); };
+            auto logit_mfmas = [&](uint32_t ks_addr, floatx16 c) -> floatx16 {
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
-                    const bf16x8 ka = *(const bf16x8*)(Ks + ln * C::KS + kk * 16 + hf * 8);
+                    const bf16x8 ka = lds_read_bf16x8(ks_addr + k_lane + kk * KKB);
                     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], c, 0, 0, 0);
                 }
                 return c;
             };
-            auto value_mfmas = [&](const uint16_t* Vt, const bf16x8* w) {
+            // all transposed V operand reads of a tile (opaque reads, settled before use)
+            auto issue_v = [&](uint32_t vt_addr, lds_half_operand (&vh)[4 * C::DT]) {
+                lds_tr_issue<0 * DTB + 0 * (16 / C::RPW) * C::GROUP, 0 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[0], vh[1]);
+                lds_tr_issue<0 * DTB + (16 / C::RPW) * C::GROUP, 0 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[2], vh[3]);
+                lds_tr_issue<1 * DTB + 0, 1 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[4], vh[5]);
+                lds_tr_issue<1 * DTB + (16 / C::RPW) * C::GROUP, 1 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[6], vh[7]);
+                if constexpr (C::DT == 4) {
+                    lds_tr_issue<2 * DTB + 0, 2 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[8], vh[9]);
+                    lds_tr_issue<2 * DTB + (16 / C::RPW) * C::GROUP, 2 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[10], vh[11]);
+                    lds_tr_issue<3 * DTB + 0, 3 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[12], vh[13]);
+                    lds_tr_issue<3 * DTB + (16 / C::RPW) * C::GROUP, 3 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[14], vh[15]);
+                }
+            };
+            auto value_mfmas = [&](uint32_t vt_addr, const bf16x8* w) {
+                lds_half_operand vh[4 * C::DT];
+                issue_v(vt_addr, vh);
+                lds_settle(vh);
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
-                        const bf16x8 va = lds_column_operand(Vt + dt * 32, C::VS, ks, lane);
+                        const bf16x8 va = lds_join(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
                         racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, w[ks], racc[dt], 0, 0, 0);
                     }
             };
@@ -340,7 +368,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 // ---- repair pass: the reference point follows the maxima on every tile ----
                 for (int s = 0; s < nt; ++s) {
                     const int j0 = (jt_lo + s) * TJ;
-                    const uint16_t* Ks = smem + buf * C::STAGE;
+                    begin_step(s);
+                    const uint32_t Ks = stage_addr(buf);
                     const bool plain = tile_plain(s);
                     const int hi = i - j0 - 4 * hf, lo = hi - w1;
                     floatx16 t;
@@ -371,7 +400,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     float rs;
                     weights(t, pb, rs);
                     l += rs;
-                    value_mfmas(Ks + C::K_ELEMS, pb);
+                    value_mfmas(Ks + C::TILE_BYTES + v_lane, pb);
                     advance();
                 }
             } else {
@@ -384,7 +413,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     floatx16 t;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) t[v] = 0.f;
-                    t = logit_mfmas(smem + buf * C::STAGE, t);
+                    t = logit_mfmas(stage_addr(buf), t);
                     float mx = -INFINITY;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
@@ -404,16 +433,18 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 floatx16 sh_a, sh_b;
                 {
                     const floatx16 c0 = tile_plain(0) ? negm : masked_c(jt_lo * TJ);
-                    sh_a = logit_mfmas(smem + buf * C::STAGE, c0);
+                    begin_step(0);
+                    sh_a = logit_mfmas(stage_addr(buf), c0);
                 }
-                uint32_t vt_prev = smem_addr + (uint32_t)(buf * C::STAGE + C::K_ELEMS) * 2u + v_lane;
+                uint32_t vt_prev = stage_addr(buf) + (uint32_t)C::TILE_BYTES + v_lane;
                 advance();
                 // One step: logits of tile s into `cur`, weights and value MFMAs of tile s-1 from `prev`.
                 auto step = [&](int s, const floatx16& prev, floatx16& cur) {
-                    const uint32_t ks_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u;
+                    begin_step(s);
+                    const uint32_t ks_addr = stage_addr(buf);
                     bf16x8 ka[C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + k_lane + kk * 32);
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + k_lane + kk * KKB);
                     // the reference point (and, on the two window-edge tiles, the mask) is the
                     // C operand of the first logit MFMA
                     if (__builtin_expect(tile_plain(s), 1)) {
@@ -422,11 +453,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                         asm volatile("" ::: "memory");      // keep the mask arithmetic out of the common path
                         cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
                     }
-                    bf16x8 va[C::DT][2];
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                        for (int ks = 0; ks < 2; ++ks) va[dt][ks] = lds_column_operand_at<C::VS>(vt_prev + dt * 64, ks);
+                    lds_half_operand vh[4 * C::DT];
+                    issue_v(vt_prev, vh);
                     bf16x8 pb[2];
                     float rs;
 #pragma unroll
@@ -435,19 +463,20 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     weights(prev, pb, rs);
                     l += rs;
                     bad |= !(rs < OVERFLOW_LIMIT);
+                    lds_settle(vh);
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) {
-                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
+                            const bf16x8 va = lds_join(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
+                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[ks], racc[dt], 0, 0, 0);
                         }
 #pragma unroll
                     for (int x = 1; x < C::DK; ++x) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
                         __builtin_amdgcn_sched_group_barrier(0x402, 5, 0);               // a slice of VALU / exp
-                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);               // two V operand reads
                     }
-                    vt_prev = ks_addr + (uint32_t)C::K_ELEMS * 2u + v_lane;
+                    vt_prev = ks_addr + (uint32_t)C::TILE_BYTES + v_lane;
                     advance();
                 };
                 int s = 1;
@@ -465,13 +494,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 }
                 l += rs;
                 bad |= !(rs < OVERFLOW_LIMIT);
-#pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const bf16x8 va = lds_column_operand_at<C::VS>(vt_prev + dt * 64, ks);
-                        racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[ks], racc[dt], 0, 0, 0);
-                    }
+                value_mfmas(vt_prev - v_lane + v_lane, pb);
             }
         }
 
@@ -510,10 +533,9 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         }
         const uint16_t* vrow = v2src + (int64_t)(ok ? vr : 0) * v2stride + 4 * hf_m;
         auto slab_of = [&](int w) -> uint16_t* {
-            if (w < 4) return slabs + w * (BQ * C::SS);
-            int fb = buf + 1 + ((w - 4) >> 1);                 // the two stage buffers other than buf
-            fb = fb >= C::NSTAGE ? fb - C::NSTAGE : fb;
-            return smem + fb * C::STAGE + ((w - 4) & 1) * (BQ * C::SS);
+            if (w < 2) return slabs + w * (BQ * C::SS);
+            const int fb = (buf + 1 + ((w - 2) >> 1)) & (C::NSTAGE - 1);      // the three stages other than buf
+            return smem + fb * C::STAGE + ((w - 2) & 1) * (BQ * C::SS);
         };
         {
             uint16_t* srow = slab_of(wave) + ln_m * C::SS + 4 * hf_m;
