@@ -43,10 +43,7 @@ WORKLOADS = {
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 547.4e6,      # 371.4 MB read + 176.0 MB written
-    ("c4", "backward"): 13280.8e6,   # rowdot + row + finalize + column kernels, reads + writes
-}
+MEASURED_TRAFFIC_BYTES = {}
 
 
 def count_triples(B, N, H, w1, w2):
@@ -187,28 +184,36 @@ def main():
     bwd_rest_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2,
                                                           needs=(True, False, True, False, True)), ksteps, 2) - rowdot_ms
     mfma = bool(lib.sa2_uses_mfma(B, N, H, D, w1, w2, _lib.SA2_BF16))
+    # Algorithmic flops per launch: forward 4*D*T; the backward's 12*D*T split evenly between its
+    # two MFMA kernels (each owns two output contractions, 4*D*T, and half of the S / dP
+    # recomputation that the pair shares, 2*D*T).
+    half_bwd = bwd_flops / 2
     kernels = {
-        "forward": {"ms": fwd_ms, "tflops": fwd_flops / fwd_ms / 1e9, "hbm_gbs": fwd_bytes / fwd_ms / 1e6},
-        "backward": {"ms": bwd_all_ms, "tflops": bwd_flops / bwd_all_ms / 1e9, "hbm_gbs": bwd_bytes / bwd_all_ms / 1e6},
-        "backward_dk_dv": {"ms": bwd_k1_ms},
-        "backward_dq_dk2_dv2": {"ms": bwd_rest_ms},
-        "rowdot": {"ms": rowdot_ms, "hbm_gbs": (4 * E + 4 * B * H * N) / rowdot_ms / 1e6},
+        "forward": {"kernel": "mfma_fwd_kernel<%d,false> (+ repair launch)" % D, "ms": fwd_ms, "flops": fwd_flops},
+        "backward_k_side": {"kernel": "mfma_bwd_kv_kernel<%d> (dK, dV)" % D, "ms": bwd_k1_ms, "flops": half_bwd},
+        "backward_kprime_side": {"kernel": "mfma_bwd_kp_kernel<%d> + dq_sum (dQ, dK', dV')" % D, "ms": bwd_rest_ms,
+                                 "flops": half_bwd},
     }
-    for k in ("forward", "backward"):
-        kernels[k]["frac_bf16_peak"] = kernels[k]["tflops"] / PEAK_BF16_TFLOPS
+    for k in kernels.values():
+        k["tflops"] = k["flops"] / k["ms"] / 1e9
+        k["frac_bf16_peak"] = k["tflops"] / PEAK_BF16_TFLOPS
+    kernels["forward"]["hbm_gbs"] = fwd_bytes / fwd_ms / 1e6
+    kernels["backward"] = {"ms": bwd_all_ms, "tflops": bwd_flops / bwd_all_ms / 1e9, "hbm_gbs": bwd_bytes / bwd_all_ms / 1e6,
+                           "frac_bf16_peak": bwd_flops / bwd_all_ms / 1e9 / PEAK_BF16_TFLOPS}
+    kernels["rowdot"] = {"ms": rowdot_ms, "hbm_gbs": (4 * E + 4 * B * H * N) / rowdot_ms / 1e6}
 
-    # The forward kernel is one launch; its duration is the forward call's.
-    dominant = "forward" if fwd_ms >= bwd_all_ms else "backward"
+    # the dominant kernel: the longest of the three MFMA kernels
+    dominant = max(("forward", "backward_k_side", "backward_kprime_side"), key=lambda k: kernels[k]["ms"])
     roofline = {
-        "bound": "mfma", "kernel": "mfma_fwd_kernel<%d>" % D if dominant == "forward" else "backward kernels (sum)",
+        "bound": "mfma", "kernel": kernels[dominant]["kernel"],
         "achieved": kernels[dominant]["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-        "frac": kernels[dominant]["tflops"] / PEAK_BF16_TFLOPS,
+        "frac": kernels[dominant]["frac_bf16_peak"],
         "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dominant)),
-        "algorithmic_flops_per_launch": fwd_flops if dominant == "forward" else bwd_flops,
+        "algorithmic_flops_per_launch": kernels[dominant]["flops"],
         "avg_ms": kernels[dominant]["ms"],
     }
     roofline_fwd = {
-        "bound": "mfma", "kernel": "mfma_fwd_kernel<%d>" % D, "achieved": kernels["forward"]["tflops"],
+        "bound": "mfma", "kernel": kernels["forward"]["kernel"], "achieved": kernels["forward"]["tflops"],
         "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": kernels["forward"]["frac_bf16_peak"],
         "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "forward")),
         "hbm_gbs": kernels["forward"]["hbm_gbs"], "hbm_frac": kernels["forward"]["hbm_gbs"] / PEAK_HBM_GBS,
