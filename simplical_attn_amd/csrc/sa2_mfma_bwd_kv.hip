@@ -31,16 +31,18 @@ struct KvCfg {
     static constexpr int TILE = BQ * TS;
     static constexpr int UNIT = 2 * TILE;      // Q~ tile, then dO~ tile
     static constexpr int NUNIT = 3;
-    static constexpr int RS = D + 8;           // raw row stride (bf16)
+    static constexpr int RS = D + 8;           // K'/V' row stride (bf16)
+    static constexpr int FS = D + 4;           // q / dO row stride (fp32)
     static constexpr int PX_BYTES = VPAIR * 2 * 64 * 32;
     static constexpr size_t LDS_LIMIT = 160 * 1024;
     static size_t lds_bytes(int w2) {
-        return (size_t)NUNIT * UNIT * 2 + PX_BYTES + 2 * BQ * RS * 2 + 2 * (size_t)(BQ + w2) * RS * 2 + 4 * BQ * 4;
+        return (size_t)NUNIT * UNIT * 2 + PX_BYTES + 2 * BQ * FS * 4 + 2 * (size_t)(BQ + w2) * RS * 2 + 4 * BQ * 4;
     }
     static bool fits(int w2) { return lds_bytes(w2) <= LDS_LIMIT; }
 };
 
-template <int D>
+// BIAS = false: k2_bias and v2_bias are both zero (the reference's default), the adds drop out.
+template <int D, bool BIAS>
 __global__ __launch_bounds__(VT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     using C = KvCfg<D>;
@@ -49,9 +51,9 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     const int SR = BQ + w2;                                   // K'/V' rows kept per query block
     uint16_t* units = (uint16_t*)smem_raw;
     unsigned char* px = smem_raw + (size_t)C::NUNIT * C::UNIT * 2;
-    uint16_t* q_s = (uint16_t*)(px + C::PX_BYTES);            // [BQ][RS]
-    uint16_t* do_s = q_s + BQ * C::RS;                        // [BQ][RS]
-    uint16_t* k2_s = do_s + BQ * C::RS;                       // [SR][RS] rows i0-w2 .. i0+31
+    float* q_s = (float*)(px + C::PX_BYTES);                  // [BQ][FS] q * scale*log2(e), fp32
+    float* do_s = q_s + BQ * C::FS;                           // [BQ][FS] dO, fp32
+    uint16_t* k2_s = (uint16_t*)(do_s + BQ * C::FS);          // [SR][RS] rows i0-w2 .. i0+31
     uint16_t* v2_s = k2_s + SR * C::RS;                       // [SR][RS]
     float* lse_s = (float*)(v2_s + SR * C::RS);               // [2][BQ]  -LSE*log2(e), by parity of ib
     float* dsum_s = lse_s + 2 * BQ;                           // [2][BQ]  -D_i
@@ -106,8 +108,14 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             const int row = c / CPR, col = c - row * CPR;
             int i = i0 + row;
             i = i < N ? i : N - 1;
-            *(uint4*)(q_s + row * C::RS + col * 8) = *(const uint4*)(qp + (int64_t)i * p.q.sn + col * 8);
-            *(uint4*)(do_s + row * C::RS + col * 8) = *(const uint4*)(dop + (int64_t)i * p.dout.sn + col * 8);
+            const uint4 qa = *(const uint4*)(qp + (int64_t)i * p.q.sn + col * 8);
+            const uint4 da = *(const uint4*)(dop + (int64_t)i * p.dout.sn + col * 8);
+            float* qd = q_s + row * C::FS + col * 8;
+            float* dd = do_s + row * C::FS + col * 8;
+            *(float4*)qd = make_float4(bf16_lo(qa.x) * qscale, bf16_hi(qa.x) * qscale, bf16_lo(qa.y) * qscale, bf16_hi(qa.y) * qscale);
+            *(float4*)(qd + 4) = make_float4(bf16_lo(qa.z) * qscale, bf16_hi(qa.z) * qscale, bf16_lo(qa.w) * qscale, bf16_hi(qa.w) * qscale);
+            *(float4*)dd = make_float4(bf16_lo(da.x), bf16_hi(da.x), bf16_lo(da.y), bf16_hi(da.y));
+            *(float4*)(dd + 4) = make_float4(bf16_lo(da.z), bf16_hi(da.z), bf16_lo(da.w), bf16_hi(da.w));
         }
         for (int c = tid; c < SR * CPR; c += VT) {
             const int row = c / CPR, col = c - row * CPR;
@@ -129,19 +137,28 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
         if (tid >= BQ * CPR) return;
         const int row = tid / CPR, col = tid - row * CPR;
         const int kr = row - delta + w2;
-        const uint4 qa = *(const uint4*)(q_s + row * C::RS + col * 8);
+        const float4 q0 = *(const float4*)(q_s + row * C::FS + col * 8), q1 = *(const float4*)(q_s + row * C::FS + col * 8 + 4);
+        const float4 d0 = *(const float4*)(do_s + row * C::FS + col * 8), d1 = *(const float4*)(do_s + row * C::FS + col * 8 + 4);
         const uint4 kx = *(const uint4*)(k2_s + kr * C::RS + col * 8);
-        const uint4 da = *(const uint4*)(do_s + row * C::RS + col * 8);
         const uint4 vx = *(const uint4*)(v2_s + kr * C::RS + col * 8);
-        const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w}, kw[4] = {kx.x, kx.y, kx.z, kx.w};
-        const uint32_t dw[4] = {da.x, da.y, da.z, da.w}, vw[4] = {vx.x, vx.y, vx.z, vx.w};
+        const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const float dv[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+        const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w}, vw[4] = {vx.x, vx.y, vx.z, vx.w};
+        const float kb = BIAS ? p.k2_bias : 0.f, vb = BIAS ? p.v2_bias : 0.f;
         bf16x8 r, d;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
-            r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
-            d[2 * t] = (__bf16)(bf16_lo(dw[t]) * (bf16_lo(vw[t]) + p.v2_bias));
-            d[2 * t + 1] = (__bf16)(bf16_hi(dw[t]) * (bf16_hi(vw[t]) + p.v2_bias));
+            if (BIAS) {
+                r[2 * t] = (__bf16)(qv[2 * t] * (bf16_lo(kw[t]) + kb));
+                r[2 * t + 1] = (__bf16)(qv[2 * t + 1] * (bf16_hi(kw[t]) + kb));
+                d[2 * t] = (__bf16)(dv[2 * t] * (bf16_lo(vw[t]) + vb));
+                d[2 * t + 1] = (__bf16)(dv[2 * t + 1] * (bf16_hi(vw[t]) + vb));
+            } else {
+                r[2 * t] = (__bf16)(qv[2 * t] * bf16_lo(kw[t]));
+                r[2 * t + 1] = (__bf16)(qv[2 * t + 1] * bf16_hi(kw[t]));
+                d[2 * t] = (__bf16)(dv[2 * t] * bf16_lo(vw[t]));
+                d[2 * t + 1] = (__bf16)(dv[2 * t + 1] * bf16_hi(vw[t]));
+            }
         }
         uint16_t* dst = units + slot * C::UNIT + row * C::TS + col * 8;
         *(bf16x8*)dst = r;
@@ -332,10 +349,12 @@ int launch_kv(const Problem& p, hipStream_t st) {
     const int64_t total = (int64_t)njb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
     const size_t lds = C::lds_bytes(p.w2);
-    if (hipFuncSetAttribute((const void*)mfma_bwd_kv_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess)
+    const bool bias = p.k2_bias != 0.f || p.v2_bias != 0.f;
+    const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<D, true> : (const void*)mfma_bwd_kv_kernel<D, false>;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL(mfma_bwd_kv_kernel<D>, dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
+    if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<D, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
+    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<D, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
 
