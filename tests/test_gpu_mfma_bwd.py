@@ -44,19 +44,30 @@ def test_small_shapes_vs_oracle(case):
                          atol=floor if name in ("dq", "dk1", "dk2") else 1e-6)
 
 
-def check_large(B, N, H, D, w1, w2, seed, rows, qk_mag=None):
+def check_rows(got, inp, w1, w2, rows):
+    """Oracle gradients of the loss restricted to query rows [r0, r1): complete for dq on those
+    rows, and for K (K') rows whose whole forward reach [j, j+w] lies inside the range or is cut
+    off by the end of the sequence."""
+    r0, r1 = rows
+    N = inp[0].shape[1]
+    want = oracle_all(inp, w1, w2, dtype=torch.float32, rows=rows)
+    assert_close_rel(got["out"][:, r0:r1], want["out"], BF16_TOL, "out rows %s" % (rows,))
+    assert_close_rel(got["dq"][:, r0:r1], want["dq"][:, r0:r1], BF16_TOL, "dq rows %s" % (rows,))
+    for name, w in (("dk1", w1), ("dv1", w1), ("dk2", w2), ("dv2", w2)):
+        hi = r1 if r1 == N else r1 - w
+        assert hi > r0
+        assert_close_rel(got[name][:, r0:hi], want[name][:, r0:hi], BF16_TOL, "%s rows %s" % (name, rows))
+
+
+def check_large(B, N, H, D, w1, w2, seed, rows, qk_mag=None, more_rows=(), generic=True):
     inp = make_inputs(B, N, H, D, seed=seed, dtype=torch.bfloat16, qk_mag=qk_mag)
     got = run_device(inp, w1, w2, flags=MFMA)
-    r0, r1 = rows
-    want = oracle_all(inp, w1, w2, dtype=torch.float32, rows=rows)
-    assert_close_rel(got["out"][:, r0:r1], want["out"], BF16_TOL, "out")
-    assert_close_rel(got["dq"][:, r0:r1], want["dq"][:, r0:r1], BF16_TOL, "dq")
-    for name, w in (("dk1", w1), ("dv1", w1), ("dk2", w2), ("dv2", w2)):
-        assert r1 - w > r0
-        assert_close_rel(got[name][:, r0:r1 - w], want[name][:, r0:r1 - w], BF16_TOL, name)
-    ref = run_device(inp, w1, w2, flags=GENERIC)
-    for name in GRADS:
-        assert_close_rel(got[name], ref[name].float().cpu(), BF16_TOL, name + " vs generic kernels")
+    for r in (rows,) + tuple(more_rows):
+        check_rows(got, inp, w1, w2, r)
+    if generic:
+        ref = run_device(inp, w1, w2, flags=GENERIC)
+        for name in GRADS:
+            assert_close_rel(got[name], ref[name].float().cpu(), BF16_TOL, name + " vs generic kernels")
 
 
 def test_config3_forward_backward():
@@ -67,6 +78,14 @@ def test_config3_forward_backward():
 def test_config4_headline_shape_gradients():
     """BASELINE config 4: bf16, B1 H16 N8192 D128, w 512/32, seed 3."""
     check_large(1, 8192, 16, 128, 512, 32, seed=3, rows=(448, 1088))
+
+
+def test_config5_long_sequence_gradients():
+    """BASELINE config 5: bf16, B1 H8 N32768 D128, w 1024/64, q/k/k' ~ N(0, 0.5^2), seed 4.  Checked
+    on query rows around i = w1 and at the end of the sequence (the generic kernels would take
+    minutes at this size)."""
+    check_large(1, 32768, 8, 128, 1024, 64, seed=4, rows=(992, 2048), qk_mag=0.5,
+                more_rows=((32768 - 320, 32768),), generic=False)
 
 
 def test_needs_input_grad_subsets_and_determinism():
