@@ -50,27 +50,33 @@ struct KpCfg {
     static constexpr int PX_BYTES = NPAIR * 2 * 64 * 32;         // P hand-over, double buffered
     static_assert(2 * BQ * RS <= STAGE, "two slabs must fit one stage buffer");
     static constexpr size_t LDS_LIMIT = 160 * 1024;
-    static size_t main_bytes(int w2) {
+    // raw = true: the q and dO rows the workgroup touches are copied to LDS; otherwise the
+    // wavefronts read them from global memory once per unit
+    static size_t main_bytes(int w2, bool raw) {
         const size_t rq = BQ + w2;
-        return (size_t)NSTAGE * STAGE * 2 + PX_BYTES + 2 * rq * RS * 2 + 2 * BQ * RS * 2 + 2 * ((rq + 3) / 4 * 4) * 4 + rq * AS * 4;
+        return (size_t)NSTAGE * STAGE * 2 + PX_BYTES + (raw ? 2 * rq * RS * 2 : 0) + 2 * BQ * RS * 2 +
+               2 * ((rq + 3) / 4 * 4) * 4 + rq * AS * 4;
     }
     static size_t final_bytes() { return (size_t)KW * BQ * AS * 4; }
-    static size_t lds_bytes(int w2) { return main_bytes(w2) > final_bytes() ? main_bytes(w2) : final_bytes(); }
-    static bool fits(int w2) { return lds_bytes(w2) <= LDS_LIMIT; }
+    static size_t lds_bytes(int w2, bool raw) {
+        return main_bytes(w2, raw) > final_bytes() ? main_bytes(w2, raw) : final_bytes();
+    }
+    static bool raw_fits(int w2) { return lds_bytes(w2, true) <= LDS_LIMIT; }
+    static bool fits(int w2) { return lds_bytes(w2, false) <= LDS_LIMIT; }
 };
 
 template <int D>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) {
+void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int raw) {
     using C = KpCfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int RQ = BQ + w2;                                   // query rows this workgroup touches
     uint16_t* smem = (uint16_t*)smem_raw;                     // stage ring
     unsigned char* px = smem_raw + (size_t)C::NSTAGE * C::STAGE * 2;
-    uint16_t* q_s = (uint16_t*)(px + C::PX_BYTES);            // [RQ][RS] q rows k0 ..
-    uint16_t* do_s = q_s + RQ * C::RS;                        // [RQ][RS] dO rows
-    uint16_t* k2_s = do_s + RQ * C::RS;                       // [BQ][RS] K' rows k0 ..
+    uint16_t* q_s = (uint16_t*)(px + C::PX_BYTES);            // [RQ][RS] q rows k0 .. (when raw)
+    uint16_t* do_s = q_s + RQ * C::RS;                        // [RQ][RS] dO rows      (when raw)
+    uint16_t* k2_s = raw ? do_s + RQ * C::RS : q_s;           // [BQ][RS] K' rows k0 ..
     uint16_t* v2_s = k2_s + BQ * C::RS;                       // [BQ][RS] V' rows
     const int RQ4 = (RQ + 3) & ~3;
     float* lse_s = (float*)(v2_s + BQ * C::RS);               // [RQ] LSE * log2(e)
@@ -135,7 +141,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     // ---- raw rows, LSE, D and the dQ accumulator -------------------------------------
     {
         constexpr int CPR = D / 8;
-        for (int c = tid; c < RQ * CPR; c += KT) {
+        for (int c = tid; c < (raw ? RQ * CPR : 0); c += KT) {
             const int row = c / CPR, col = c - row * CPR;
             int r = k0 + row;
             r = r < N ? r : N - 1;
@@ -158,6 +164,17 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         for (int c = tid; c < RQ * C::AS; c += KT) dqacc[c] = 0.f;
     }
 
+    // q / dO row of query k0 + rel: the LDS copy or (clamped) global memory
+    auto q_row = [&](int rel) -> const uint16_t* {
+        if (raw) return q_s + rel * C::RS;
+        const int r = k0 + rel < N ? k0 + rel : N - 1;
+        return qp + (int64_t)r * p.q.sn;
+    };
+    auto do_row = [&](int rel) -> const uint16_t* {
+        if (raw) return do_s + rel * C::RS;
+        const int r = k0 + rel < N ? k0 + rel : N - 1;
+        return dop + (int64_t)r * p.dout.sn;
+    };
     const float qscale = p.scale * LOG2E;
     const uint32_t smem_addr = lds_address(smem);
     const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * 64 * 32 + lane * 32);
@@ -246,7 +263,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             bf16x8 qf[C::DK];
             float lse2 = 0.f;
             {
-                const uint16_t* qrow = q_s + (ln + delta) * C::RS + hf * 8;
+                const uint16_t* qrow = q_row(ln + delta) + hf * 8;
                 const uint16_t* krow = k2_s + ln * C::RS + hf * 8;
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
@@ -320,7 +337,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             }
             // dV'[k] += R[(k+delta, k)] * dO[k+delta]
             if (ok) {
-                const uint16_t* drow = do_s + (ln + delta) * C::RS + 4 * hf;
+                const uint16_t* drow = do_row(ln + delta) + 4 * hf;
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -356,7 +373,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             bf16x8 dof[C::DK];
             float dsum = 0.f;
             {
-                const uint16_t* drow = do_s + (ln + delta) * C::RS + hf * 8;
+                const uint16_t* drow = do_row(ln + delta) + hf * 8;
                 const uint16_t* vrow = v2_s + ln * C::RS + hf * 8;
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
@@ -421,7 +438,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             if (nt - 1 >= sa && nt - 1 <= sb) consume();
             // dK'[k] += G[(k+delta, k)] * q[k+delta]   (scale applied at the end)
             if (ok) {
-                const uint16_t* qrow = q_s + (ln + delta) * C::RS + 4 * hf;
+                const uint16_t* qrow = q_row(ln + delta) + 4 * hf;
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -554,12 +571,13 @@ int launch_kp(const Problem& p, hipStream_t st) {
     const int64_t total = (int64_t)nkb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
     if (p.dq.p && p.scratch_bytes < kp_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
-    const size_t lds = C::lds_bytes(p.w2);
+    const int raw = C::raw_fits(p.w2) ? 1 : 0;
+    const size_t lds = C::lds_bytes(p.w2, raw != 0);
     if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
     float* part = (float*)p.scratch;
-    hipLaunchKernelGGL(mfma_bwd_kp_kernel<D>, dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part);
+    hipLaunchKernelGGL(mfma_bwd_kp_kernel<D>, dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, raw);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (p.dq.p) {
         const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
