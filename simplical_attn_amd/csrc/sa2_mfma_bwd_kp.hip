@@ -40,11 +40,15 @@ template <int D>
 struct KpCfg {
     static constexpr int DK = D / 16;
     static constexpr int DT = D / 32;
-    static constexpr int TS = D + 24;          // K/V tile row stride (bf16): full-rate row reads, good transpose reads
-    static constexpr int TILE = TJ * TS;
-    static constexpr int STAGE = 2 * TILE;     // K tile, then V tile
+    // K and V tiles are written by direct global->LDS loads: one wavefront instruction fills a
+    // group of RPW rows (1 KB), lane L putting the 16-byte chunk L / RPW of row L % RPW at byte
+    // 16 * L; groups lie GROUP bytes apart.  Row and transposed operand reads are conflict free.
+    static constexpr int RPW = 512 / D;
+    static constexpr int GROUP = 1024 + 16 * RPW;
+    static constexpr int NGROUP = TJ / RPW;
+    static constexpr int TILE_BYTES = NGROUP * GROUP;
+    static constexpr int STAGE = TILE_BYTES;   // bf16 elements of a stage: K tile, then V tile
     static constexpr int NSTAGE = 3;
-    static constexpr int KCH = TJ * D / 8;     // 16-byte chunks per tile
     static constexpr int RS = D + 8;           // raw row / slab row stride (bf16)
     static constexpr int AS = D + 4;           // fp32 accumulator row stride
     static constexpr int PX_BYTES = NPAIR * 2 * 64 * 32;         // P hand-over, double buffered
@@ -110,14 +114,14 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const int total_steps = nrounds * nt;
     const bool want_dq = p.dq.p != nullptr;
 
-    // ---- staging of one K/V tile: global -> registers -> LDS (one K and one V chunk per thread)
-    const bool t_owner = tid < C::KCH;
-    const int t_row = tid / (D / 8), t_col = tid - t_row * (D / 8);
+    // ---- staging of one K/V tile: wavefront w requests group w of both tiles, straight into LDS
+    const bool t_owner = wave < C::NGROUP;
+    const int t_row = wave * C::RPW + (lane % C::RPW), t_col = lane / C::RPW;
     const uint32_t k_off = ((uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8) * 2u;
     const uint32_t v_off = ((uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8) * 2u;
-    uint16_t* st_dst = smem + t_row * C::TS + t_col * 8;
-    uint4 kreg = make_uint4(0u, 0u, 0u, 0u), vreg = make_uint4(0u, 0u, 0u, 0u);
-    auto load_tile = [&](int jt) {
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    typedef const __attribute__((address_space(1))) void* glb_ptr;
+    auto dma_tile = [&](int jt, int stage) {
         const int j0 = jt * TJ;
         if (!t_owner) return;
         uint32_t ko = k_off, vo = v_off;
@@ -128,14 +132,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         }
         const char* kbp = (const char*)(k1p + (int64_t)j0 * p.k1.sn);
         const char* vbp = (const char*)(v1p + (int64_t)j0 * p.v1.sn);
-        kreg = *(const uint4*)(kbp + ko);
-        vreg = *(const uint4*)(vbp + vo);
-    };
-    auto store_tile = [&](int sb) {
-        if (!t_owner) return;
-        uint16_t* Ks = st_dst + sb * C::STAGE;
-        *(uint4*)Ks = kreg;
-        *(uint4*)(Ks + C::TILE) = vreg;
+        unsigned char* dst = smem_raw + (size_t)stage * (C::STAGE * 2) + wave * C::GROUP;
+        __builtin_amdgcn_global_load_lds((glb_ptr)(kbp + ko), (lds_ptr)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((glb_ptr)(vbp + vo), (lds_ptr)(dst + C::TILE_BYTES), 16, 0, 0);
     };
 
     // ---- raw rows, LSE, D and the dQ accumulator -------------------------------------
@@ -178,23 +177,38 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const float qscale = p.scale * LOG2E;
     const uint32_t smem_addr = lds_address(smem);
     const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * 64 * 32 + lane * 32);
-    const uint32_t row_lane = (uint32_t)(ln * C::TS + hf * 8) * 2u;          // row operand: row ln, k-slots of this half
-    const uint32_t col_lane = lds_column_lane_offset(C::TS, lane);           // transposed operand
+    const uint32_t row_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);   // row operand
+    const uint32_t col_lane = lds_group_column_lane_offset<C::RPW, C::GROUP>(lane);                      // transposed operand
+    constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;      // operand strides of a k-step / a 32-column block
+    constexpr uint32_t GA = (16 / C::RPW) * C::GROUP, GB = (8 / C::RPW) * C::GROUP;
+    // all transposed operand reads of a tile (opaque reads, settled before use)
+    auto issue_tr = [&](uint32_t a, lds_half_operand (&h)[4 * C::DT]) {
+        lds_tr_issue<0, GB>(a, h[0], h[1]);
+        lds_tr_issue<GA, GA + GB>(a, h[2], h[3]);
+        lds_tr_issue<DTB, DTB + GB>(a, h[4], h[5]);
+        lds_tr_issue<DTB + GA, DTB + GA + GB>(a, h[6], h[7]);
+        if constexpr (C::DT == 4) {
+            lds_tr_issue<2 * DTB, 2 * DTB + GB>(a, h[8], h[9]);
+            lds_tr_issue<2 * DTB + GA, 2 * DTB + GA + GB>(a, h[10], h[11]);
+            lds_tr_issue<3 * DTB, 3 * DTB + GB>(a, h[12], h[13]);
+            lds_tr_issue<3 * DTB + GA, 3 * DTB + GA + GB>(a, h[14], h[15]);
+        }
+    };
 
-    load_tile(jt_lo);
-    store_tile(0);
-    if (total_steps > 1) load_tile(jt_lo + (1 % nt));
-    int next_tile = 2 % nt;
+    dma_tile(jt_lo, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    int g = 0, buf = 0;
-    auto advance = [&]() {
-        const int nb = buf + 1 == C::NSTAGE ? 0 : buf + 1;
-        if (g + 1 < total_steps) store_tile(nb);
-        if (g + 2 < total_steps) load_tile(jt_lo + next_tile);
+    // Step g works on ring stage g % 3 (the dS wavefronts also on the one before).  The tile of
+    // step g+1 is requested at the start of step g and must have landed at its end.
+    int g = 0, buf = 0, next_tile = 1 % nt;
+    auto begin_step = [&]() {
+        if (g + 1 < total_steps) dma_tile(jt_lo + next_tile, buf + 1 == C::NSTAGE ? 0 : buf + 1);
         next_tile = next_tile + 1 == nt ? 0 : next_tile + 1;
-        __syncthreads();
-        buf = nb;
+    };
+    auto advance = [&]() {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        buf = buf + 1 == C::NSTAGE ? 0 : buf + 1;
         ++g;
     };
 
@@ -282,12 +296,13 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 if (ok) lse2 = lse_s[ln + delta];
             }
             for (int s = 0; s < nt; ++s) {
+                begin_step();
                 if (s >= sa && s <= sb) {
                     const int j0 = (jt_lo + s) * TJ;
                     const uint32_t ks_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u;
                     bf16x8 ka[C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + row_lane + kk * 32);
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + row_lane + kk * KKB);
                     floatx16 sh;
                     const bool plain = rows_full && j0 + TJ - 1 <= i_min && j0 >= i_max - w1;
                     if (__builtin_expect(plain, 1)) {
@@ -315,23 +330,20 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
                         for (int t = 0; t < 8; ++t) pb[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t] - lse2);
+                    lds_half_operand vh[4 * C::DT];
+                    issue_tr(ks_addr + (uint32_t)C::TILE_BYTES + col_lane, vh);
                     {
-                        typedef bf16x8 __attribute__((address_space(3)))* lds_b8;
+                        // opaque stores: the compiler would wait for the tile request in flight
                         const uint32_t a = px_addr + (uint32_t)((g & 1) * 64 * 32);
-                        *(lds_b8)(uintptr_t)a = pb[0];
-                        *(lds_b8)(uintptr_t)(a + 16) = pb[1];
+                        asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16" ::"v"(a), "v"(pb[0]), "v"(pb[1]) : "memory");
                     }
-                    const uint32_t vt_addr = ks_addr + (uint32_t)C::TILE * 2u + col_lane;
-                    bf16x8 va[C::DT][2];
-#pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                        for (int ks = 0; ks < 2; ++ks) va[dt][ks] = lds_column_operand_at<C::TS>(vt_addr + dt * 64, ks);
+                    lds_settle(vh);
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks)
-                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][ks], pb[ks], racc[dt], 0, 0, 0);
+                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_join(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]),
+                                                                               pb[ks], racc[dt], 0, 0, 0);
                 }
                 advance();
             }
@@ -400,12 +412,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 const uint32_t a = px_addr + (uint32_t)(((g - 1) & 1) * 64 * 32);
                 const bf16x8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
                 const int pb = buf == 0 ? C::NSTAGE - 1 : buf - 1;
-                const uint32_t kt_addr = smem_addr + (uint32_t)(pb * C::STAGE) * 2u + col_lane;
-                bf16x8 kt[C::DT][2];
-#pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) kt[dt][ks] = lds_column_operand_at<C::TS>(kt_addr + dt * 64, ks);
+                lds_half_operand kh[4 * C::DT];
+                issue_tr(smem_addr + (uint32_t)(pb * C::STAGE) * 2u + col_lane, kh);
+                lds_settle(kh);
                 bf16x8 dsb[2];
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
@@ -416,18 +425,20 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
-                        gacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt[dt][ks], dsb[ks], gacc[dt], 0, 0, 0);
+                        gacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_join(kh[4 * dt + 2 * ks], kh[4 * dt + 2 * ks + 1]),
+                                                                           dsb[ks], gacc[dt], 0, 0, 0);
             };
             for (int s = 0; s < nt; ++s) {
+                begin_step();
                 floatx16 dp;
                 const bool act = s >= sa && s <= sb;
                 if (act) {
-                    const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE + C::TILE) * 2u;
+                    const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u + (uint32_t)C::TILE_BYTES;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) dp[v] = 0.f;
 #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) {
-                        const bf16x8 va = lds_read_bf16x8(vs_addr + row_lane + kk * 32);
+                        const bf16x8 va = lds_read_bf16x8(vs_addr + row_lane + kk * KKB);
                         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp, 0, 0, 0);
                     }
                 }
