@@ -43,7 +43,11 @@ WORKLOADS = {
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    ("c4", "forward"): 379.5e6,                # 345.4 MB read + 34.1 MB written
+    ("c4", "backward_k_side"): 628.0e6,        # 560.9 MB read + 67.1 MB written
+    ("c4", "backward_kprime_side"): 908.3e6,   # kernel 405.4 + 201.3 MB, dq_sum 268.0 + 33.6 MB
+}
 
 
 def count_triples(B, N, H, w1, w2):
