@@ -295,6 +295,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 }
                 if (ok) lse2 = lse_s[ln + delta];
             }
+            floatx16 negl;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) negl[v] = -lse2;
             for (int s = 0; s < nt; ++s) {
                 begin_step();
                 if (s >= sa && s <= sb) {
@@ -306,10 +309,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     floatx16 sh;
                     const bool plain = rows_full && j0 + TJ - 1 <= i_min && j0 >= i_max - w1;
                     if (__builtin_expect(plain, 1)) {
-                        floatx16 zero;
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) zero[v] = 0.f;
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], zero, 0, 0, 0);
+                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], negl, 0, 0, 0);
                     } else {
                         asm volatile("" ::: "memory");
                         // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
@@ -318,7 +318,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int c = 8 * (v >> 2) + (v & 3);
-                            ct[v] = (row_ok & (c <= hi) & (c >= lo)) ? 0.f : -INFINITY;
+                            ct[v] = (row_ok & (c <= hi) & (c >= lo)) ? negl[0] : -INFINITY;
                         }
                         sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], ct, 0, 0, 0);
                     }
@@ -329,7 +329,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                        for (int t = 0; t < 8; ++t) pb[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t] - lse2);
+                        for (int t = 0; t < 8; ++t) pb[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t]);
                     lds_half_operand vh[4 * C::DT];
                     issue_tr(ks_addr + (uint32_t)C::TILE_BYTES + col_lane, vh);
                     {
@@ -403,9 +403,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 }
                 if (ok) dsum = dsum_s[ln + delta];
             }
-            floatx16 dp_prev;
+            floatx16 dp_prev, negd;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) dp_prev[v] = 0.f;
+            for (int v = 0; v < 16; ++v) { dp_prev[v] = 0.f; negd[v] = -dsum; }
             // dS of the tile handled in the previous step and its G MFMAs
             auto consume = [&]() {
                 typedef const bf16x8 __attribute__((address_space(3)))* lds_b8;
@@ -418,8 +418,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 bf16x8 dsb[2];
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    dsb[0][t] = (__bf16)((float)p0[t] * (dp_prev[t] - dsum));
-                    dsb[1][t] = (__bf16)((float)p1[t] * (dp_prev[8 + t] - dsum));
+                    dsb[0][t] = (__bf16)((float)p0[t] * dp_prev[t]);
+                    dsb[1][t] = (__bf16)((float)p1[t] * dp_prev[8 + t]);
                 }
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
@@ -430,20 +430,19 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             };
             for (int s = 0; s < nt; ++s) {
                 begin_step();
-                floatx16 dp;
-                const bool act = s >= sa && s <= sb;
-                if (act) {
-                    const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u + (uint32_t)C::TILE_BYTES;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) dp[v] = 0.f;
-#pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) {
-                        const bf16x8 va = lds_read_bf16x8(vs_addr + row_lane + kk * KKB);
-                        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp, 0, 0, 0);
-                    }
-                }
                 if (s - 1 >= sa && s - 1 <= sb) consume();
-                if (act) dp_prev = dp;
+                if (s >= sa && s <= sb) {
+                    const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u + (uint32_t)C::TILE_BYTES;
+                    bf16x8 va[C::DK];
+#pragma unroll
+                    for (int kk = 0; kk < C::DK; ++kk) va[kk] = lds_read_bf16x8(vs_addr + row_lane + kk * KKB);
+                    dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[0], dof[0], negd, 0, 0, 0);
+#pragma unroll
+                    for (int kk = 1; kk < C::DK; ++kk)
+                        dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[kk], dof[kk], dp_prev, 0, 0, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
+                }
                 advance();
             }
             if (nt - 1 >= sa && nt - 1 <= sb) consume();
