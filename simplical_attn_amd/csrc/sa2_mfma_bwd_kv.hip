@@ -279,18 +279,20 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                             oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[dt][ks], pb[ks], oacc[dt], 0, 0, 0);
                 }
             } else {
-                floatx16 dp;
+                // first the previous unit (its dP is still in dp_prev), then this unit's dP
+                if (act_prev) consume(slot == 0 ? C::NUNIT - 1 : slot - 1, step - 1);
                 if (act) {
                     const uint32_t d_addr = u_addr + (uint32_t)C::TILE * 2u;
-                    dp = negr;
+                    bf16x8 da[C::DK];
     #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) {
-                        const bf16x8 da = lds_read_bf16x8(d_addr + row_lane + kk * 32);
-                        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, kvf[kk], dp, 0, 0, 0);
-                    }
+                    for (int kk = 0; kk < C::DK; ++kk) da[kk] = lds_read_bf16x8(d_addr + row_lane + kk * 32);
+                    dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[0], kvf[0], negr, 0, 0, 0);
+    #pragma unroll
+                    for (int kk = 1; kk < C::DK; ++kk)
+                        dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[kk], kvf[kk], dp_prev, 0, 0, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
                 }
-                if (act_prev) consume(slot == 0 ? C::NUNIT - 1 : slot - 1, step - 1);
-                if (act) dp_prev = dp;
                 act_prev = act;
             }
 
