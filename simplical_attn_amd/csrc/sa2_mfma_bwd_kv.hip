@@ -132,17 +132,26 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
         }
     };
     // ---- form unit (ib, delta) into a ring slot: one 16-byte chunk of Q~ and of dO~ per thread ----
+    // this thread's chunk of the block's q and dO rows stays in registers for the block's units
+    float qv[8], dv[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) qv[t] = dv[t] = 0.f;
+    auto fetch_qd = [&]() {
+        constexpr int CPR = D / 8;
+        if (tid >= BQ * CPR) return;
+        const int row = tid / CPR, col = tid - row * CPR;
+        const float4 q0 = *(const float4*)(q_s + row * C::FS + col * 8), q1 = *(const float4*)(q_s + row * C::FS + col * 8 + 4);
+        const float4 d0 = *(const float4*)(do_s + row * C::FS + col * 8), d1 = *(const float4*)(do_s + row * C::FS + col * 8 + 4);
+        qv[0] = q0.x; qv[1] = q0.y; qv[2] = q0.z; qv[3] = q0.w; qv[4] = q1.x; qv[5] = q1.y; qv[6] = q1.z; qv[7] = q1.w;
+        dv[0] = d0.x; dv[1] = d0.y; dv[2] = d0.z; dv[3] = d0.w; dv[4] = d1.x; dv[5] = d1.y; dv[6] = d1.z; dv[7] = d1.w;
+    };
     auto form = [&](int delta, int slot) {
         constexpr int CPR = D / 8;
         if (tid >= BQ * CPR) return;
         const int row = tid / CPR, col = tid - row * CPR;
         const int kr = row - delta + w2;
-        const float4 q0 = *(const float4*)(q_s + row * C::FS + col * 8), q1 = *(const float4*)(q_s + row * C::FS + col * 8 + 4);
-        const float4 d0 = *(const float4*)(do_s + row * C::FS + col * 8), d1 = *(const float4*)(do_s + row * C::FS + col * 8 + 4);
         const uint4 kx = *(const uint4*)(k2_s + kr * C::RS + col * 8);
         const uint4 vx = *(const uint4*)(v2_s + kr * C::RS + col * 8);
-        const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-        const float dv[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
         const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w}, vw[4] = {vx.x, vx.y, vx.z, vx.w};
         const float kb = BIAS ? p.k2_bias : 0.f, vb = BIAS ? p.v2_bias : 0.f;
         bf16x8 r, d;
@@ -173,6 +182,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     // ---- prologue: first block's raw rows, first unit --------------------------------
     load_raw(ib_lo);
     __syncthreads();
+    fetch_qd();
     form(0, 0);
     __syncthreads();
 
@@ -309,6 +319,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                     __syncthreads();         // nobody still forms from the old rows
                     load_raw(nib);
                     __syncthreads();
+                    fetch_qd();
                     nu = units_of(nib);
                 }
                 form(ndelta, nslot);
