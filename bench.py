@@ -44,9 +44,9 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 379.5e6,                # 345.4 MB read + 34.1 MB written
-    ("c4", "backward_k_side"): 628.0e6,        # 560.9 MB read + 67.1 MB written
-    ("c4", "backward_kprime_side"): 908.3e6,   # kernel 405.4 + 201.3 MB, dq_sum 268.0 + 33.6 MB
+    ("c4", "forward"): 380.2e6,                # reads + writes of the forward kernel
+    ("c4", "backward_k_side"): 620.2e6,        # mfma_bwd_kv_kernel
+    ("c4", "backward_kprime_side"): 933.3e6,   # mfma_bwd_kp_kernel 631.8 MB + dq_sum 301.5 MB
 }
 
 
