@@ -8,7 +8,10 @@ from .simplicial_attn import (  # noqa: F401
     simplicial_forward,
 )
 
+from .compiled_op import two_simplicial_attention  # noqa: F401,E402
+
 __all__ = [
+    "two_simplicial_attention",
     "TwoSimplicialAttention",
     "TwoSimplicialAttentionFunction",
     "compute_D_kernel",
