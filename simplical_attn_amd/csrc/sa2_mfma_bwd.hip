@@ -1,9 +1,11 @@
-// bf16 MFMA backward for gfx950, head_dim 64 or 128.
+// bf16 MFMA backward for gfx950, head_dim 64 or 128: dispatch, and the workspace kernels
+// that serve shapes whose K' window is too wide for the on-chip kernels
+// (sa2_mfma_bwd_kp.hip for dQ, dK', dV'; sa2_mfma_bwd_kv.hip for dK, dV).
 //
 // Same expanded-row view as the forward: rows r = (i, delta), Q~[r] = q[i] *
 // k2~[i-delta] * scale*log2(e) and dO~[r] = dO[i] * v2~[i-delta], both bf16.  With
 // P = exp2(S - LSE*log2e) recomputed from the saved log-sum-exp and
-// dS = P * (dO~.v1 - D_i):
+// dS = P * (dO~.v1 - D_i), the workspace kernels are:
 //
 //   row kernel      owns 32 queries x one delta per wavefront, sweeps the K window:
 //                   G[r,:] = scale * sum_j dS[r,j] k1[j,:]   and   R[r,:] = sum_j P[r,j] v1[j,:]

@@ -13,7 +13,6 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 constexpr int BQ = 32;       // queries per workgroup
 constexpr int TJ = 32;       // keys per LDS tile
 constexpr int NTHREADS = 256;
-constexpr float RESCALE_LOG2 = 8.0f;
 constexpr float OVERFLOW_LIMIT = 1.0e30f;    // a row sum above this means a stale softmax reference point
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
@@ -129,23 +128,6 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 __device__ __forceinline__ bf16x8 lds_read_bf16x8(uint32_t addr) {
     return *(const bf16x8 __attribute__((address_space(3)))*)(uintptr_t)addr;
 }
-
-// acc *= alpha for an MFMA accumulator that lives in AGPRs, without asking the
-// register allocator for a VGPR copy of the tuple (it would place that copy on
-// the hot path).  Used only on the rare rescale path; the s_nop before the
-// first read covers the MFMA-write -> VALU-read distance, the one after the
-// last write the VALU-write -> MFMA-read distance.
-__device__ __forceinline__ void scale_acc(floatx16& acc, float alpha) {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        float x = acc[v], t;
-        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
-                     : "+a"(x), "=&v"(t)
-                     : "v"(alpha));
-        acc[v] = x;
-    }
-}
-
 
 }  // namespace
 }  // namespace sa2

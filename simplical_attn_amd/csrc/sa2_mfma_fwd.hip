@@ -13,10 +13,11 @@
 // wavefront's softmax arithmetic overlaps the other's MFMAs) owns 32 consecutive
 // queries of one (batch, head).  A "unit" is (delta, those 32 queries) = one
 // 32-row MFMA N-tile; each wavefront holds one unit at a time and sweeps the K
-// window [i0-w1, i0+31] in 32-key tiles that the workgroup stages through a
-// three-deep LDS ring, both row-major; K operands are 16-byte LDS reads, V
-// operands come out of LDS transposed (ds_read_b64_tr_b16).  The q rows of the block and the K'/V'
-// rows its deltas reach are copied to LDS once.  On unmasked tiles each step
+// window [i0-w1, i0+31] in 32-key tiles that go straight from global memory into a
+// four-stage LDS ring (global_load_lds, two steps ahead of their use) in a grouped
+// layout that both the 16-byte K operand reads and the transposed V operand reads
+// (ds_read_b64_tr_b16) take without bank conflicts.  The q rows of the block and the
+// K'/V' rows its deltas reach are copied to LDS once.  On unmasked tiles each step
 // issues the logit MFMAs of tile t between the softmax instructions of tile t-1
 // and then the value MFMAs of tile t-1, so neither pipe waits for the other inside
 // the one barrier interval per tile.  After each round of 8 units the wavefronts fold their
@@ -521,7 +522,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln_m] * fast_exp2(xch_m[w * BQ + ln_m] - Muse);
         if (wave == 0 && hf_m == 0) xch_a[ln_m] = a;
         // Every wavefront writes its contribution c * (v2 + bias) * R as bf16 into its own
-        // slab: four slabs have their own LDS, the other four use the two stage buffers
+        // slab: two slabs have their own LDS, the other six use the three stage buffers
         // that hold no live tile between rounds.  Then every thread adds its slice of the
         // eight slabs in wavefront order.
         const float cw = ok ? fast_exp2(m - Muse) : 0.f;
