@@ -22,6 +22,8 @@
 //       G^T += K1^T.dS^T.
 // Every MFMA operand that streams from LDS is read once per 32x32x16 MFMA; transposed
 // operands come from the row-major tiles through ds_read_b64_tr_b16.
+#include <type_traits>
+
 #include "sa2_mfma_common.h"
 
 namespace sa2 {
@@ -52,7 +54,6 @@ struct KpCfg {
     static constexpr int RS = D + 8;           // raw row / slab row stride (bf16)
     static constexpr int AS = D + 4;           // fp32 accumulator row stride
     static constexpr int PX_BYTES = NPAIR * 2 * 64 * 32;         // P hand-over, double buffered
-    static_assert(2 * BQ * RS <= STAGE, "two slabs must fit one stage buffer");
     static constexpr size_t LDS_LIMIT = 160 * 1024;
     // raw = true: the q and dO rows the workgroup touches are copied to LDS; otherwise the
     // wavefronts read them from global memory once per unit
@@ -69,9 +70,12 @@ struct KpCfg {
     static bool fits(int w2) { return lds_bytes(w2, false) <= LDS_LIMIT; }
 };
 
-template <int D>
+// RAW = true: the q and dO rows the workgroup touches are copied to LDS; otherwise the
+// wavefronts read them from global memory once per unit.
+template <int D, bool RAW>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int raw) {
+void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) {
+    constexpr bool raw = RAW;
     using C = KpCfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
@@ -111,7 +115,17 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const int nt = jt_hi - jt_lo + 1;
     const int n_units = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1;
     const int nrounds = (n_units + NPAIR - 1) / NPAIR;
-    const int total_steps = nrounds * nt;
+    // Tiles a round sweeps: from the first tile of its smallest delta to the last tile of its
+    // largest one (tile indices relative to jt_lo).
+    auto round_first = [&](int round) {
+        const int i_min = k0 + round * NPAIR;
+        return (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo;
+    };
+    auto round_last = [&](int round) {
+        const int dl = (round + 1) * NPAIR - 1 < n_units - 1 ? (round + 1) * NPAIR - 1 : n_units - 1;
+        const int i_max = k0 + dl + BQ - 1 < N - 1 ? k0 + dl + BQ - 1 : N - 1;
+        return i_max / TJ - jt_lo;
+    };
     const bool want_dq = p.dq.p != nullptr;
 
     // ---- staging of one K/V tile: wavefront w requests group w of both tiles, straight into LDS
@@ -164,15 +178,21 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     }
 
     // q / dO row of query k0 + rel: the LDS copy or (clamped) global memory
-    auto q_row = [&](int rel) -> const uint16_t* {
-        if (raw) return q_s + rel * C::RS;
-        const int r = k0 + rel < N ? k0 + rel : N - 1;
-        return qp + (int64_t)r * p.q.sn;
+    auto q_row = [&](int rel) {
+        if constexpr (RAW) {
+            return (const uint16_t*)(q_s + rel * C::RS);
+        } else {
+            const int r = k0 + rel < N ? k0 + rel : N - 1;
+            return qp + (int64_t)r * p.q.sn;
+        }
     };
-    auto do_row = [&](int rel) -> const uint16_t* {
-        if (raw) return do_s + rel * C::RS;
-        const int r = k0 + rel < N ? k0 + rel : N - 1;
-        return dop + (int64_t)r * p.dout.sn;
+    auto do_row = [&](int rel) {
+        if constexpr (RAW) {
+            return (const uint16_t*)(do_s + rel * C::RS);
+        } else {
+            const int r = k0 + rel < N ? k0 + rel : N - 1;
+            return dop + (int64_t)r * p.dout.sn;
+        }
     };
     const float qscale = p.scale * LOG2E;
     const uint32_t smem_addr = lds_address(smem);
@@ -195,17 +215,25 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         }
     };
 
-    dma_tile(jt_lo, 0);
+    // Step g works on ring stage g % 3 (the dS wavefronts also on the one before).  The tile of
+    // step g+1 (the next one of this round, or the first one of the next round) is requested at
+    // the start of step g and must have landed at its end.
+    int g = 0, buf = 0;
+    int next_round = 0, next_tile = round_first(0), next_last = round_last(0);
+    auto next_request = [&](int stage) {
+        if (next_round < nrounds) dma_tile(jt_lo + next_tile, stage);
+        if (next_tile == next_last) {
+            ++next_round;
+            next_tile = round_first(next_round);
+            next_last = round_last(next_round);
+        } else {
+            ++next_tile;
+        }
+    };
+    next_request(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-
-    // Step g works on ring stage g % 3 (the dS wavefronts also on the one before).  The tile of
-    // step g+1 is requested at the start of step g and must have landed at its end.
-    int g = 0, buf = 0, next_tile = 1 % nt;
-    auto begin_step = [&]() {
-        if (g + 1 < total_steps) dma_tile(jt_lo + next_tile, buf + 1 == C::NSTAGE ? 0 : buf + 1);
-        next_tile = next_tile + 1 == nt ? 0 : next_tile + 1;
-    };
+    auto begin_step = [&]() { next_request(buf + 1 == C::NSTAGE ? 0 : buf + 1); };
     auto advance = [&]() {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         buf = buf + 1 == C::NSTAGE ? 0 : buf + 1;
@@ -218,44 +246,6 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) pacc[dt][v] = 0.f;
-
-    // slab of pair w for the dQ merge: the two stage buffers other than `buf`
-    auto slab_of = [&](int w) -> uint16_t* {
-        int fb = buf + 1 + (w >> 1);
-        fb = fb >= C::NSTAGE ? fb - C::NSTAGE : fb;
-        return smem + fb * C::STAGE + (w & 1) * (BQ * C::RS);
-    };
-    // add the round's four slabs (rows shifted by their delta) into the dQ accumulator
-    auto merge_dq = [&](int round) {
-        const int tid_m = kp_recompute_here(threadIdx.x);
-        constexpr int CH = D / 16;
-        for (int it = tid_m; it < RQ * CH; it += KT) {
-            const int row = it / CH, c0 = (it - row * CH) * 16;
-            float acc[16];
-#pragma unroll
-            for (int c = 0; c < 16; ++c) acc[c] = 0.f;
-#pragma unroll
-            for (int w = 0; w < NPAIR; ++w) {
-                const int dl = round * NPAIR + w;
-                const int kl = row - dl;
-                if (dl < n_units && kl >= 0 && kl < BQ) {
-                    const uint16_t* sp = slab_of(w) + kl * C::RS + c0;
-                    const uint4 x = *(const uint4*)sp, y = *(const uint4*)(sp + 8);
-                    acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
-                    acc[4] += bf16_lo(x.z); acc[5] += bf16_hi(x.z); acc[6] += bf16_lo(x.w); acc[7] += bf16_hi(x.w);
-                    acc[8] += bf16_lo(y.x); acc[9] += bf16_hi(y.x); acc[10] += bf16_lo(y.y); acc[11] += bf16_hi(y.y);
-                    acc[12] += bf16_lo(y.z); acc[13] += bf16_hi(y.z); acc[14] += bf16_lo(y.w); acc[15] += bf16_hi(y.w);
-                }
-            }
-            float* ap = dqacc + row * C::AS + c0;
-#pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
-                float4 a = *(float4*)(ap + 4 * c4);
-                a.x += acc[4 * c4]; a.y += acc[4 * c4 + 1]; a.z += acc[4 * c4 + 2]; a.w += acc[4 * c4 + 3];
-                *(float4*)(ap + 4 * c4) = a;
-            }
-        }
-    };
 
     if (role == 0) {
         // =============================== P wavefronts ================================
@@ -298,7 +288,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             floatx16 negl;
 #pragma unroll
             for (int v = 0; v < 16; ++v) negl[v] = -lse2;
-            for (int s = 0; s < nt; ++s) {
+            const int s_end = round_last(round);
+            for (int s = round_first(round); s <= s_end; ++s) {
                 begin_step();
                 if (s >= sa && s <= sb) {
                     const int j0 = (jt_lo + s) * TJ;
@@ -362,10 +353,10 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     }
             }
             if (want_dq) {
-                __syncthreads();       // the dS wavefronts are done with the last tile
-                __syncthreads();       // slabs written
-                merge_dq(round);
-                __syncthreads();       // the stage buffers that served as slabs are free again
+                // the dS wavefronts add their dQ contributions in four phases
+                __syncthreads();
+                __syncthreads();
+                __syncthreads();
             }
         }
     } else {
@@ -428,7 +419,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                         gacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_join(kh[4 * dt + 2 * ks], kh[4 * dt + 2 * ks + 1]),
                                                                            dsb[ks], gacc[dt], 0, 0, 0);
             };
-            for (int s = 0; s < nt; ++s) {
+            const int s_end = round_last(round);
+            for (int s = round_first(round); s <= s_end; ++s) {
                 begin_step();
                 if (s - 1 >= sa && s - 1 <= sb) consume();
                 if (s >= sa && s <= sb) {
@@ -445,7 +437,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 }
                 advance();
             }
-            if (nt - 1 >= sa && nt - 1 <= sb) consume();
+            if (s_end >= sa && s_end <= sb) consume();
             // dK'[k] += G[(k+delta, k)] * q[k+delta]   (scale applied at the end)
             if (ok) {
                 const uint16_t* qrow = q_row(ln + delta) + 4 * hf;
@@ -461,27 +453,58 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     }
             }
             if (want_dq) {
-                __syncthreads();       // every dS wavefront is done with the last tile
-                if (ok) {
-                    // dQ contribution of the unit: scale * G * k2~, row ln of the slab is query k0+ln+delta
-                    uint16_t* srow = slab_of(pr) + ln * C::RS + 4 * hf;
-                    const uint16_t* krow = k2_s + ln * C::RS + 4 * hf;
+                // dQ contribution of the unit: dqacc[ln + delta][:] += G * k2~.  The four dS
+                // wavefronts add into the shared fp32 accumulator (scale is applied when the
+                // partial is written out) in four phases; in phase t
+                // wavefront pr owns the 16-column blocks (pr + t) % 4 (and that + 4 when D = 128),
+                // so no two wavefronts touch an element at the same time and every element
+                // receives its contributions in a fixed order.
+                auto add_dq = [&](auto PR, auto BIASED) {
+                    constexpr int P0 = decltype(PR)::value;
+                    constexpr bool WITH_BIAS = decltype(BIASED)::value;
+                    const int tid_q = kp_recompute_here(threadIdx.x);
+                    const int ln_q = tid_q & 31, hf_q = (tid_q >> 5) & 1;
+                    float* arow = dqacc + (ln_q + delta) * C::AS + 4 * hf_q;
+                    const uint16_t* krow = k2_s + ln_q * C::RS + 4 * hf_q;
 #pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
+                    for (int t = 0; t < 4; ++t) {
+                        if (ok) {
+                            constexpr int NV = C::DK / 2;             // float4 slots of this phase
+                            float4 a[NV];
+                            uint2 x[NV];
 #pragma unroll
-                        for (int g4 = 0; g4 < 4; ++g4) {
-                            const uint2 x = *(const uint2*)(krow + dt * 32 + 8 * g4);
-                            union { __bf16 h[4]; uint2 u; } o;
-                            o.h[0] = (__bf16)(p.scale * gacc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.k2_bias));
-                            o.h[1] = (__bf16)(p.scale * gacc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.k2_bias));
-                            o.h[2] = (__bf16)(p.scale * gacc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.k2_bias));
-                            o.h[3] = (__bf16)(p.scale * gacc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.k2_bias));
-                            *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
+                            for (int e = 0; e < NV; ++e) {
+                                const int sb16 = ((P0 + t) & 3) + 4 * (e >> 1);
+                                const int col = (sb16 >> 1) * 32 + 8 * (2 * (sb16 & 1) + (e & 1));
+                                x[e] = *(const uint2*)(krow + col);
+                                a[e] = *(float4*)(arow + col);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int e = 0; e < NV; ++e) {
+                                const int sb16 = ((P0 + t) & 3) + 4 * (e >> 1);
+                                const int dt = sb16 >> 1, g4 = 2 * (sb16 & 1) + (e & 1);
+                                const float kb = WITH_BIAS ? p.k2_bias : 0.f;
+                                a[e].x += gacc[dt][4 * g4 + 0] * (bf16_lo(x[e].x) + kb);
+                                a[e].y += gacc[dt][4 * g4 + 1] * (bf16_hi(x[e].x) + kb);
+                                a[e].z += gacc[dt][4 * g4 + 2] * (bf16_lo(x[e].y) + kb);
+                                a[e].w += gacc[dt][4 * g4 + 3] * (bf16_hi(x[e].y) + kb);
+                                *(float4*)(arow + (sb16 >> 1) * 32 + 8 * g4) = a[e];
+                            }
                         }
-                }
-                __syncthreads();
-                merge_dq(round);
-                __syncthreads();
+                        if (t < 3) __syncthreads();
+                    }
+                };
+                auto add_dq_of = [&](auto BIASED) {
+                    switch (pr) {
+                        case 0: add_dq(std::integral_constant<int, 0>{}, BIASED); break;
+                        case 1: add_dq(std::integral_constant<int, 1>{}, BIASED); break;
+                        case 2: add_dq(std::integral_constant<int, 2>{}, BIASED); break;
+                        default: add_dq(std::integral_constant<int, 3>{}, BIASED); break;
+                    }
+                };
+                if (p.k2_bias != 0.f) add_dq_of(std::true_type{});
+                else add_dq_of(std::false_type{});
             }
         }
     }
@@ -494,7 +517,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         float* dst = dq_part + ((int64_t)bh * nkb + kb) * RQ * D;
         for (int it = tid_f; it < RQ * CH; it += KT) {
             const int row = it / CH, c0 = (it - row * CH) * 4;
-            *(float4*)(dst + (int64_t)row * D + c0) = *(const float4*)(dqacc + row * C::AS + c0);
+            float4 a = *(const float4*)(dqacc + row * C::AS + c0);
+            a.x *= p.scale; a.y *= p.scale; a.z *= p.scale; a.w *= p.scale;
+            *(float4*)(dst + (int64_t)row * D + c0) = a;
         }
     }
     __syncthreads();
@@ -581,13 +606,14 @@ int launch_kp(const Problem& p, hipStream_t st) {
     const int64_t total = (int64_t)nkb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
     if (p.dq.p && p.scratch_bytes < kp_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
-    const int raw = C::raw_fits(p.w2) ? 1 : 0;
-    const size_t lds = C::lds_bytes(p.w2, raw != 0);
-    if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess)
-        return SA2_ERR_LAUNCH_FAILED;
+    const bool raw = C::raw_fits(p.w2);
+    const size_t lds = C::lds_bytes(p.w2, raw);
     float* part = (float*)p.scratch;
-    hipLaunchKernelGGL(mfma_bwd_kp_kernel<D>, dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, raw);
+    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<D, true> : (const void*)mfma_bwd_kp_kernel<D, false>;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return SA2_ERR_LAUNCH_FAILED;
+    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, true>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part);
+    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (p.dq.p) {
         const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
