@@ -29,6 +29,8 @@
 // R^T = V^T . P^T.  The softmax reference point of a unit is fixed at the first
 // tile that holds one of its keys and enters the logit MFMA as its C operand, so
 // on unmasked tiles the vector ALU only does exp2, bf16 packing and a row sum.
+#include <type_traits>
+
 #include "sa2_mfma_common.h"
 
 namespace sa2 {
@@ -63,7 +65,7 @@ struct Cfg {
     // LDS carve-up (bytes)
     static constexpr int NSTAGE = 4;
     static constexpr size_t STAGE_BYTES = (size_t)NSTAGE * STAGE * 2;
-    static constexpr size_t SLAB_BYTES = (size_t)2 * BQ * SS * 2;          // two slabs; six more live in idle stage buffers
+    static constexpr size_t SLAB_BYTES = (size_t)3 * BQ * SS * 2;          // three slabs; four more live in idle stage buffers
     static_assert(2 * BQ * SS <= STAGE, "two slabs must fit one stage buffer");
     static constexpr size_t OACC_BYTES = (size_t)BQ * OS * 4;
     static constexpr size_t XCH_BYTES = (size_t)(2 * FW * BQ + 3 * BQ) * 4;
@@ -92,8 +94,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     float* oacc = (float*)(smem_raw + C::STAGE_BYTES + C::SLAB_BYTES);
     float* xch_m = oacc + BQ * C::OS;           // [FW][BQ]
     float* xch_l = xch_m + FW * BQ;             // [FW][BQ]
-    float* xch_a = xch_l + FW * BQ;             // [BQ] accumulator rescale of this round
-    float* fin_m = xch_a + BQ;                  // [BQ] final M
+    float* fin_m = xch_l + FW * BQ + BQ;        // [BQ] final M
     float* fin_l = fin_m + BQ;                  // [BQ] final L
     uint16_t* q_s = (uint16_t*)(fin_l + BQ);    // [BQ][KS] q rows of the block
     uint16_t* k2_s = q_s + BQ * C::KS;          // [BQ + w2][KS] K' rows i0-w2 .. i0+31 (when side_kv)
@@ -178,6 +179,11 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     }
     bool bad = false;
 
+    // the first two tiles are requested before anything else so that their latency overlaps
+    // the copies below
+    dma_next();
+    if (total_steps > 1) dma_next();
+
     // ---- q rows of the block and the K'/V' rows its deltas reach, once, to LDS ----
     const int side_rows = BQ + w2;
     uint16_t* v2_s = k2_s + side_rows * C::KS;
@@ -216,10 +222,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     const uint32_t k_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);
     const uint32_t v_lane = lds_group_column_lane_offset<C::RPW, C::GROUP>(lane);
 
-    dma_next();
-    if (total_steps > 1) dma_next();
-    if (total_steps > 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     // Tiles [s_lo, s_hi] need no mask: every key of the tile is inside the K window of
@@ -229,14 +232,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     const int s_hi = (i0 + 1) / TJ - 1 - jt_lo;                 // last tile with j0+31 <= i0
 
     // Step g of the sweep works on ring stage g % NSTAGE.  At its start the tile of step g+2 is
-    // requested (the stage it goes to was last read in step g-1); at its end the tile of step
-    // g+1 must have landed.  The last step of a round requests nothing, so that three stages
-    // are free for the merge; the first step of the next round catches up.
+    // requested (the stage it goes to was last read in step g-2); at its end the tile of step
+    // g+1 must have landed.  Requests run on across rounds, so between two rounds the ring
+    // holds the first tile of the next round, has its second one in flight, and two stages
+    // are free for the merge.
     int g = 0, buf = 0;                                         // buf = g % NSTAGE
     bool requested = false;
-    auto begin_step = [&](int s) {
-        if (s == 0 && g > 0 && dma_count < total_steps) dma_next();
-        requested = s + 1 < nt && dma_count < total_steps;
+    auto begin_step = [&](int) {
+        requested = dma_count < total_steps;
         if (requested) dma_next();
     };
     auto advance = [&]() {
@@ -270,20 +273,25 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
             {
                 const uint16_t* krow = k2src + (int64_t)side_row(delta) * k2stride + hf * 8;
                 const uint16_t* qrow = q_s + ln * C::KS + hf * 8;
+                auto form_q = [&](auto BIASED) {
+                    const float kbias = decltype(BIASED)::value ? p.k2_bias : 0.f;
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) {
-                    const uint4 qa = *(const uint4*)(qrow + kk * 16);
-                    const uint4 kb = *(const uint4*)(krow + kk * 16);
-                    const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
-                    const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
-                    bf16x8 r;
+                    for (int kk = 0; kk < C::DK; ++kk) {
+                        const uint4 qa = *(const uint4*)(qrow + kk * 16);
+                        const uint4 kb = *(const uint4*)(krow + kk * 16);
+                        const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
+                        const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
+                        bf16x8 r;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
-                        r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
+                        for (int t = 0; t < 4; ++t) {
+                            r[2 * t] = (__bf16)(bf16_lo(qw[t]) * qscale * (bf16_lo(kw[t]) + kbias));
+                            r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * qscale * (bf16_hi(kw[t]) + kbias));
+                        }
+                        qf[kk] = r;
                     }
-                    qf[kk] = r;
-                }
+                };
+                if (p.k2_bias != 0.f) form_q(std::true_type{});
+                else form_q(std::false_type{});
             }
             const bool rows_full = i0 >= delta && i0 + BQ - 1 < N;
             const bool row_ok = i < N && i >= delta;
@@ -520,11 +528,11 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         float Ln = Lrun * a;
 #pragma unroll
         for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln_m] * fast_exp2(xch_m[w * BQ + ln_m] - Muse);
-        if (wave == 0 && hf_m == 0) xch_a[ln_m] = a;
-        // Every wavefront writes its contribution c * (v2 + bias) * R as bf16 into its own
-        // slab: two slabs have their own LDS, the other six use the three stage buffers
-        // that hold no live tile between rounds.  Then every thread adds its slice of the
-        // eight slabs in wavefront order.
+        // Wavefront 0 rescales the accumulator rows by a and adds its contribution
+        // c * (v2 + bias) * R in place (its lanes own whole rows there).  Every other wavefront
+        // writes its contribution as bf16 into its own slab: three slabs have their own LDS, the
+        // other four use the two stage buffers that hold no tile of the next round.  Then
+        // every thread adds its slice of the seven slabs in wavefront order.
         const float cw = ok ? fast_exp2(m - Muse) : 0.f;
         int vr;
         if (side_kv) vr = ln_m + w2 - delta;
@@ -534,37 +542,75 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         }
         const uint16_t* vrow = v2src + (int64_t)(ok ? vr : 0) * v2stride + 4 * hf_m;
         auto slab_of = [&](int w) -> uint16_t* {
-            if (w < 2) return slabs + w * (BQ * C::SS);
-            const int fb = (buf + 1 + ((w - 2) >> 1)) & (C::NSTAGE - 1);      // the three stages other than buf
-            return smem + fb * C::STAGE + ((w - 2) & 1) * (BQ * C::SS);
+            if (w < 4) return slabs + (w - 1) * (BQ * C::SS);
+            const int fb = (buf + 2 + ((w - 4) >> 1)) & (C::NSTAGE - 1);      // the two stages after the next round's first two
+            return smem + fb * C::STAGE + (w & 1) * (BQ * C::SS);
         };
-        {
-            uint16_t* srow = slab_of(wave) + ln_m * C::SS + 4 * hf_m;
+        // PLAIN: every weight this wavefront applies is 1 (its unit started from the query's
+        // running reference point and that did not move) and there is no V' bias.
+        auto contribute = [&](auto PLAIN_TAG) {
+            constexpr bool PLAIN = decltype(PLAIN_TAG)::value;
+            const float vb = PLAIN ? 0.f : p.v2_bias;
+            if (wave == 0) {
+                float* arow = oacc + ln_m * C::OS + 4 * hf_m;
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt)
+                for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
-                    union { __bf16 h[4]; uint2 u; } o;
-                    o.h[0] = (__bf16)(cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
-                    o.h[1] = (__bf16)(cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
-                    o.h[2] = (__bf16)(cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
-                    o.h[3] = (__bf16)(cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
-                    *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
-                }
-        }
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        float4 o = *(float4*)(arow + dt * 32 + 8 * g4);
+                        if (PLAIN) {
+                            o.x += racc[dt][4 * g4 + 0] * bf16_lo(x.x);
+                            o.y += racc[dt][4 * g4 + 1] * bf16_hi(x.x);
+                            o.z += racc[dt][4 * g4 + 2] * bf16_lo(x.y);
+                            o.w += racc[dt][4 * g4 + 3] * bf16_hi(x.y);
+                        } else {
+                            o.x = o.x * a + cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + vb);
+                            o.y = o.y * a + cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + vb);
+                            o.z = o.z * a + cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + vb);
+                            o.w = o.w * a + cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + vb);
+                        }
+                        *(float4*)(arow + dt * 32 + 8 * g4) = o;
+                    }
+            } else {
+                uint16_t* srow = slab_of(wave) + ln_m * C::SS + 4 * hf_m;
+                const float c1 = PLAIN ? 1.f : cw;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        union { __bf16 h[4]; uint2 u; } o;
+                        if (PLAIN) {
+                            o.h[0] = (__bf16)(racc[dt][4 * g4 + 0] * bf16_lo(x.x));
+                            o.h[1] = (__bf16)(racc[dt][4 * g4 + 1] * bf16_hi(x.x));
+                            o.h[2] = (__bf16)(racc[dt][4 * g4 + 2] * bf16_lo(x.y));
+                            o.h[3] = (__bf16)(racc[dt][4 * g4 + 3] * bf16_hi(x.y));
+                        } else {
+                            o.h[0] = (__bf16)(c1 * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + vb));
+                            o.h[1] = (__bf16)(c1 * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + vb));
+                            o.h[2] = (__bf16)(c1 * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + vb));
+                            o.h[3] = (__bf16)(c1 * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + vb));
+                        }
+                        *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
+                    }
+            }
+        };
+        // (a unit that does not exist has cw = 0 and R = 0: it may take either path)
+        const bool plain_lane = ((a == 1.f) | (wave != 0)) & ((cw == 1.f) | !ok) & (p.v2_bias == 0.f);
+        if (__builtin_amdgcn_ballot_w64(!plain_lane) == 0) contribute(std::true_type{});
+        else contribute(std::false_type{});
         __syncthreads();
         if (wave == 0 && hf_m == 0) {
             fin_m[ln_m] = Mn;
             fin_l[ln_m] = Ln;
         }
         {
-            const float ar = xch_a[aq];
             float acc[ACN];
 #pragma unroll
-            for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c] * ar;
+            for (int c = 0; c < ACN; ++c) acc[c] = oacc[aq * C::OS + ac + c];
 #pragma unroll
-            for (int w = 0; w < FW; ++w) {
+            for (int w = 1; w < FW; ++w) {
                 const uint16_t* sp = slab_of(w) + aq * C::SS + ac;
                 if (ACN == 8) {
                     const uint4 x = *(const uint4*)sp;
@@ -579,7 +625,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
 #pragma unroll
             for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
         }
-        __syncthreads();       // the stage buffers that served as slabs are written again by the next step
+        __syncthreads();       // the stage buffers that served as slabs are requested again in the next steps
     }
 
     // ---- normalise and store ------------------------------------------------------
