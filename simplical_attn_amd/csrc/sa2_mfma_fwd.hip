@@ -84,9 +84,21 @@ struct Cfg {
 // SAFE = true: the repair kernel, launched right after: a block that finds the mark
 // recomputes itself refreshing the reference point on every tile; every other block
 // exits at once.
-template <int D, bool SAFE>
+// MODE_LEFT: the pre-pass for window sizes that leave one unit over after the rounds of
+// eight (w2 + 1 = 8n + 1).  A workgroup takes eight consecutive query blocks, one per
+// wavefront, and computes the unit delta = w2 of each while sharing one sweep of K/V tiles.
+// Nothing is merged across wavefronts: every query's partial result goes to `out` as
+// R * (v2 + bias) / l in bf16 and to `lse` as m + log2(l); the fast kernel, launched next with
+// left = 1, starts its accumulator from that pair and handles delta < w2 in full rounds.
+constexpr int MODE_FAST = 0, MODE_SAFE = 1, MODE_LEFT = 2;
+
+// SIDE: the K' and V' rows the block's deltas reach are copied to LDS (they fit); otherwise
+// they are read from global memory where they are needed.
+template <int D, int MODE, bool SIDE>
 __global__ __launch_bounds__(FT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
+void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
+    constexpr bool SAFE = MODE == MODE_SAFE, LEFT = MODE == MODE_LEFT;
+    static_assert(!(LEFT && SIDE), "the pre-pass keeps no row copies in LDS");
     using C = Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* smem = (uint16_t*)smem_raw;
@@ -94,10 +106,11 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     float* oacc = (float*)(smem_raw + C::STAGE_BYTES + C::SLAB_BYTES);
     float* xch_m = oacc + BQ * C::OS;           // [FW][BQ]
     float* xch_l = xch_m + FW * BQ;             // [FW][BQ]
-    float* fin_m = xch_l + FW * BQ + BQ;        // [BQ] final M
+    float* lam_s = xch_l + FW * BQ;             // [BQ] reference point of the pre-pass partial
+    float* fin_m = lam_s + BQ;                  // [BQ] final M
     float* fin_l = fin_m + BQ;                  // [BQ] final L
     uint16_t* q_s = (uint16_t*)(fin_l + BQ);    // [BQ][KS] q rows of the block
-    uint16_t* k2_s = q_s + BQ * C::KS;          // [BQ + w2][KS] K' rows i0-w2 .. i0+31 (when side_kv)
+    uint16_t* k2_s = q_s + BQ * C::KS;          // [BQ + w2][KS] K' rows i0-w2 .. i0+31 (when SIDE)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -108,10 +121,12 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     // K/V window) run on the same XCD and meet in its L2.
     int pid = blockIdx.x;
     if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    const int bh = pid / nqb, qb = pid - bh * nqb;
+    // (in the pre-pass nqb counts groups of eight query blocks)
+    const int bh = pid / nqb, qb = LEFT ? (pid - bh * nqb) * FW + wave : pid - bh * nqb;
     const int b = bh / p.H, h = bh - b * p.H;
     const int N = p.N, w1 = p.w1, w2 = p.w2;
-    const int i0 = qb * BQ;
+    const int i0 = qb * BQ;                      // per wavefront in the pre-pass
+    const int i0_wg = LEFT ? (qb - wave) * BQ : i0;
     const int i = i0 + ln;
     const int ic = i < N ? i : N - 1;
     const int i_last = (i0 + BQ - 1 < N ? i0 + BQ - 1 : N - 1);
@@ -126,12 +141,17 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     const uint16_t* v1p = (const uint16_t*)p.v1.p + p.v1.off(b, 0, h);
     const uint16_t* v2p = (const uint16_t*)p.v2.p + p.v2.off(b, 0, h);
 
-    const int jt_lo = (i0 - w1 > 0 ? i0 - w1 : 0) / TJ;
-    const int jt_hi = i_last / TJ;
+    const int jt_lo = (i0_wg - w1 > 0 ? i0_wg - w1 : 0) / TJ;
+    const int jt_hi = LEFT ? (i0_wg + FW * BQ - 1 < N - 1 ? i0_wg + FW * BQ - 1 : N - 1) / TJ : i_last / TJ;
     const int nt = jt_hi - jt_lo + 1;
-    const int n_units = (w2 < i_last ? w2 : i_last) + 1;     // delta = 0 .. n_units-1
+    // delta = 0 .. n_units-1; the fast kernel leaves delta = w2 to the pre-pass where that ran
+    const bool has_left = left && i_last >= w2;
+    const int n_units = LEFT ? 1 : (w2 < i_last ? w2 : i_last) + 1 - (has_left && !SAFE ? 1 : 0);
     const int nrounds = (n_units + FW - 1) / FW;
     const int total_steps = nrounds * nt;
+    // tiles of the sweep that hold keys of this wavefront's rows (the whole sweep outside the pre-pass)
+    const int ws0 = LEFT ? (i0 - w1 > 0 ? i0 - w1 : 0) / TJ - jt_lo : 0;
+    const int ws1 = LEFT ? (i_last < 0 ? 0 : i_last) / TJ - jt_lo : nt - 1;
 
     // ---- staging of one K/V tile: direct global -> LDS loads ------------------------
     // Wavefront w fills group w of the K tile and of the V tile (the first NGROUP wavefronts
@@ -167,17 +187,40 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     // ---- workgroup accumulators ------------------------------------------------
     // thread -> (query aq, ACN columns from ac) of the fp32 accumulator in LDS
     constexpr int ACN = D / 16;                    // columns per thread (8 or 4)
-    {
-        const int aq = tid >> 4, ac = (tid & 15) * ACN;
-#pragma unroll
-        for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = 0.f;
-    }
-    // running maximum and sum of every query: fin_m / fin_l in LDS, read and updated at the merges
-    if (tid < BQ) {
-        fin_m[tid] = -INFINITY;
-        fin_l[tid] = 0.f;
-    }
     bool bad = false;
+    if constexpr (!LEFT) {
+        // running maximum and sum of every query: fin_m / fin_l in LDS, read and updated at the
+        // merges.  Where the pre-pass ran the accumulator starts from its partial result, which
+        // enters the first merge with weight 1 at its own reference point m + log2 l.
+        const int aq = tid >> 4, ac = (tid & 15) * ACN;
+        const int io = i0 + aq < N ? i0 + aq : N - 1;
+        if (has_left && !SAFE) {
+            const uint16_t* prow = (const uint16_t*)p.out.p + p.out.off(b, io, h) + ac;
+            if (ACN == 8) {
+                const uint4 x = *(const uint4*)prow;
+                float* o = oacc + aq * C::OS + ac;
+                o[0] = bf16_lo(x.x); o[1] = bf16_hi(x.x); o[2] = bf16_lo(x.y); o[3] = bf16_hi(x.y);
+                o[4 % ACN] = bf16_lo(x.z); o[5 % ACN] = bf16_hi(x.z); o[6 % ACN] = bf16_lo(x.w); o[7 % ACN] = bf16_hi(x.w);
+            } else {
+                const uint2 x = *(const uint2*)prow;
+                float* o = oacc + aq * C::OS + ac;
+                o[0] = bf16_lo(x.x); o[1] = bf16_hi(x.x); o[2] = bf16_lo(x.y); o[3] = bf16_hi(x.y);
+            }
+            if (tid < BQ) {
+                const int it = i0 + tid < N ? i0 + tid : N - 1;
+                const float lam = p.lse[(int64_t)bh * N + it];
+                bad = !(lam == lam);                           // the pre-pass overflowed: repair the block
+                lam_s[tid] = lam;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = 0.f;
+        }
+        if (tid < BQ) {
+            fin_m[tid] = -INFINITY;
+            fin_l[tid] = 0.f;
+        }
+    }
 
     // the first two tiles are requested before anything else so that their latency overlaps
     // the copies below
@@ -187,7 +230,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     // ---- q rows of the block and the K'/V' rows its deltas reach, once, to LDS ----
     const int side_rows = BQ + w2;
     uint16_t* v2_s = k2_s + side_rows * C::KS;
-    {
+    if constexpr (!LEFT) {
         constexpr int CPR = D / 8;                 // 16-byte chunks per row
         for (int c = tid; c < BQ * CPR; c += FT) {
             const int row = c / CPR, col = c - row * CPR;
@@ -195,7 +238,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
             r = r < N ? r : N - 1;
             *(uint4*)(q_s + row * C::KS + col * 8) = *(const uint4*)(qp + (int64_t)r * p.q.sn + col * 8);
         }
-        if (side_kv) {
+        if constexpr (SIDE) {
             for (int c = tid; c < side_rows * CPR; c += FT) {
                 const int row = c / CPR, col = c - row * CPR;
                 int r = i0 - w2 + row;
@@ -206,13 +249,13 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         }
     }
     // K'/V' row of this lane's query for a given delta: LDS copy or global memory
-    const uint16_t* k2src = side_kv ? (const uint16_t*)k2_s : k2p;
-    const uint16_t* v2src = side_kv ? (const uint16_t*)v2_s : v2p;
-    const int64_t k2stride = side_kv ? C::KS : p.k2.sn, v2stride = side_kv ? C::KS : p.v2.sn;
-    auto side_row = [&](int delta) {
-        if (side_kv) return ln + w2 - delta;       // (i0 + ln - delta) - (i0 - w2)
-        int k = ic - delta;
-        return k > 0 ? k : 0;
+    auto k2_row = [&](int delta) {
+        if constexpr (SIDE) {
+            return (const uint16_t*)(k2_s + (ln + w2 - delta) * C::KS);       // row (i0 + ln - delta) - (i0 - w2)
+        } else {
+            const int k = ic - delta;
+            return k2p + (int64_t)(k > 0 ? k : 0) * p.k2.sn;
+        }
     };
 
     const float qscale = p.scale * LOG2E;
@@ -250,11 +293,12 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     };
 
     for (int round = 0; round < nrounds; ++round) {
-        const int delta = round * FW + wave;
-        const bool ok = delta < n_units;
+        const int delta = LEFT ? w2 : round * FW + wave;
+        const bool ok = LEFT ? (i0 < N && i_last >= w2) : delta < n_units;
         // The unit starts from the query's running reference point (finite from the second
-        // round on), so only the first round has to look for maxima.
-        float m = ok ? fin_m[ln] : -INFINITY, l = 0.f;
+        // round on, or from the first where the pre-pass ran), so only then it looks for maxima.
+        float m = -INFINITY, l = 0.f;
+        if constexpr (!LEFT) m = ok ? fin_m[ln] : -INFINITY;
         floatx16 racc[C::DT];
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
@@ -271,8 +315,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
             // ---- new unit: Q~ operand, fresh softmax state ----------------------
             bf16x8 qf[C::DK];
             {
-                const uint16_t* krow = k2src + (int64_t)side_row(delta) * k2stride + hf * 8;
-                const uint16_t* qrow = q_s + ln * C::KS + hf * 8;
+                const uint16_t* krow = k2_row(delta) + hf * 8;
+                const uint16_t* qrow;
+                if constexpr (LEFT) qrow = qp + (int64_t)ic * p.q.sn + hf * 8;
+                else qrow = q_s + ln * C::KS + hf * 8;
                 auto form_q = [&](auto BIASED) {
                     const float kbias = decltype(BIASED)::value ? p.k2_bias : 0.f;
 #pragma unroll
@@ -416,8 +462,12 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 // ---- reference point: the query's running one, or (first round) the maximum of
                 // the first tile, or 0 for a row with no key there.  Any finite reference is
                 // exact as long as no weight overflows, which `bad` watches.
+                for (int s = 0; s < ws0; ++s) {           // (pre-pass) tiles before this wavefront's window
+                    begin_step(s);
+                    advance();
+                }
                 if (__builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
-                    const int j0 = jt_lo * TJ;
+                    const int j0 = (jt_lo + ws0) * TJ;
                     const int hi = i - j0 - 4 * hf, lo = hi - w1;
                     floatx16 t;
 #pragma unroll
@@ -441,8 +491,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 // of tile t-1; the shifted logits of tile t wait in registers for step t+1.
                 floatx16 sh_a, sh_b;
                 {
-                    const floatx16 c0 = tile_plain(0) ? negm : masked_c(jt_lo * TJ);
-                    begin_step(0);
+                    const floatx16 c0 = tile_plain(ws0) ? negm : masked_c((jt_lo + ws0) * TJ);
+                    begin_step(ws0);
                     sh_a = logit_mfmas(stage_addr(buf), c0);
                 }
                 uint32_t vt_prev = stage_addr(buf) + (uint32_t)C::TILE_BYTES + v_lane;
@@ -488,14 +538,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                     vt_prev = ks_addr + (uint32_t)C::TILE_BYTES + v_lane;
                     advance();
                 };
-                int s = 1;
-                for (; s + 1 < nt; s += 2) {
+                int s = ws0 + 1;
+                for (; s + 1 <= ws1; s += 2) {
                     step(s, sh_a, sh_b);
                     step(s + 1, sh_b, sh_a);
                 }
                 bf16x8 pb[2];
                 float rs;
-                if (s < nt) {
+                if (s <= ws1) {
                     step(s, sh_a, sh_b);
                     weights(sh_b, pb, rs);
                 } else {
@@ -504,7 +554,40 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
                 l += rs;
                 bad |= !(rs < OVERFLOW_LIMIT);
                 value_mfmas(vt_prev - v_lane + v_lane, pb);
+                for (int s2 = ws1 + 1; s2 < nt; ++s2) {   // (pre-pass) tiles after this wavefront's window
+                    begin_step(s2);
+                    advance();
+                }
             }
+        }
+
+        if constexpr (LEFT) {
+            // ---- pre-pass: every wavefront stores the partial result of its own unit -------
+            const float lt = l + other_half(l);
+            const bool any_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
+            if (ok && i < N) {
+                const float inv = lt > 0.f ? 1.f / lt : 0.f;
+                const int kr = i - delta > 0 ? i - delta : 0;
+                const uint16_t* vrow = v2p + (int64_t)kr * p.v2.sn + 4 * hf;
+                uint16_t* orow = (uint16_t*)p.out.p + p.out.off(b, i, h) + 4 * hf;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        union { __bf16 h[4]; uint2 u; } o;
+                        o.h[0] = (__bf16)(inv * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
+                        o.h[1] = (__bf16)(inv * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
+                        o.h[2] = (__bf16)(inv * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
+                        o.h[3] = (__bf16)(inv * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
+                        *(uint2*)(orow + dt * 32 + 8 * g4) = o.u;
+                    }
+                if (hf == 0) {
+                    const float lam = lt > 0.f ? m + __log2f(lt) : -INFINITY;
+                    p.lse[(int64_t)bh * N + i] = any_bad ? __builtin_nanf("") : lam;
+                }
+            }
+            return;
         }
 
         // ---- fold the round's units into the workgroup accumulator --------------
@@ -519,12 +602,19 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
             xch_l[wave * BQ + ln_m] = lt;
         }
         __syncthreads();
-        const float Mrun = fin_m[ln_m], Lrun = fin_l[ln_m];
+        float Mrun = fin_m[ln_m], Lrun = fin_l[ln_m];
         float Mn = Mrun;
 #pragma unroll
         for (int w = 0; w < FW; ++w) Mn = fmaxf(Mn, xch_m[w * BQ + ln_m]);
         const float Muse = (Mn == -INFINITY) ? 0.f : Mn;
+        if (has_left && !SAFE && round == 0) {
+            // the pre-pass partial: weight 1 at its own reference point, which stays out of the
+            // running maximum (that remains the value of a logit)
+            Mrun = lam_s[ln_m];
+            Lrun = Mrun > -INFINITY ? 1.f : 0.f;
+        }
         const float a = fast_exp2(Mrun - Muse);
+        bad |= !(a < OVERFLOW_LIMIT);
         float Ln = Lrun * a;
 #pragma unroll
         for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln_m] * fast_exp2(xch_m[w * BQ + ln_m] - Muse);
@@ -534,13 +624,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
         // other four use the two stage buffers that hold no tile of the next round.  Then
         // every thread adds its slice of the seven slabs in wavefront order.
         const float cw = ok ? fast_exp2(m - Muse) : 0.f;
-        int vr;
-        if (side_kv) vr = ln_m + w2 - delta;
-        else {
+        const uint16_t* vrow;
+        if constexpr (SIDE) {
+            vrow = v2_s + (ok ? ln_m + w2 - delta : 0) * C::KS + 4 * hf_m;
+        } else {
             const int iq = i0 + ln_m < N ? i0 + ln_m : N - 1;
-            vr = iq - delta > 0 ? iq - delta : 0;
+            const int vr = ok && iq - delta > 0 ? iq - delta : 0;
+            vrow = v2p + (int64_t)vr * p.v2.sn + 4 * hf_m;
         }
-        const uint16_t* vrow = v2src + (int64_t)(ok ? vr : 0) * v2stride + 4 * hf_m;
         auto slab_of = [&](int w) -> uint16_t* {
             if (w < 4) return slabs + (w - 1) * (BQ * C::SS);
             const int fb = (buf + 2 + ((w - 4) >> 1)) & (C::NSTAGE - 1);      // the two stages after the next round's first two
@@ -651,20 +742,36 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int side_kv) {
     }
 }
 
+template <int D, bool SIDE>
+int launch_fwd_kernels(const Problem& p, int nqb, int total, hipStream_t st) {
+    using C = Cfg<D>;
+    const size_t lds = C::lds_bytes(p.w2);
+    // one unit left over after the rounds of eight: the pre-pass takes it
+    const int left = (p.w2 >= FW && p.w2 % FW == 0) ? 1 : 0;
+    if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, MODE_FAST, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess ||
+        hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, MODE_SAFE, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess ||
+        hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, MODE_LEFT, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)C::STAGE_BYTES) != hipSuccess)
+        return SA2_ERR_LAUNCH_FAILED;
+    if (left) {
+        const int ngrp = (nqb + FW - 1) / FW;
+        const int total_left = ngrp * (total / nqb);
+        hipLaunchKernelGGL((mfma_fwd_kernel<D, MODE_LEFT, false>), dim3((unsigned)total_left), dim3(FT), C::STAGE_BYTES, st, p,
+                           ngrp, total_left, 0);
+        if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    }
+    hipLaunchKernelGGL((mfma_fwd_kernel<D, MODE_FAST, SIDE>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, left);
+    if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL((mfma_fwd_kernel<D, MODE_SAFE, SIDE>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, left);
+    return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
+}
+
 template <int D>
 int launch_fwd_pair(const Problem& p, int nqb, int total, hipStream_t st) {
-    using C = Cfg<D>;
-    const int side_kv = C::side_fits(p.w2) ? 1 : 0;
-    const size_t lds = C::lds_bytes(p.w2);
-    if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess ||
-        hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess)
-        return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL((mfma_fwd_kernel<D, false>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, side_kv);
-    if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL((mfma_fwd_kernel<D, true>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, side_kv);
-    return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
+    return Cfg<D>::side_fits(p.w2) ? launch_fwd_kernels<D, true>(p, nqb, total, st)
+                                   : launch_fwd_kernels<D, false>(p, nqb, total, st);
 }
 
 bool aligned16(const Tensor& t, int B, int N, int H) {
