@@ -72,10 +72,18 @@ struct KpCfg {
 
 // RAW = true: the q and dO rows the workgroup touches are copied to LDS; otherwise the
 // wavefronts read them from global memory once per unit.
-template <int D, bool RAW>
+//
+// LEFT = true: the pre-pass for window sizes that leave one unit over after the rounds of
+// four (w2 + 1 = 4n + 1).  A workgroup takes four consecutive K' blocks, one per wavefront
+// pair, and computes the unit delta = w2 of each in one shared sweep of K/V tiles.  Its
+// results go where the main kernel (launched next with left = 1) picks them up: dK'
+// (unscaled) and dV' as bf16 in the output tensors, the dQ contribution as fp32 in rows
+// w2 .. w2+31 of the block's dQ partial.  The main kernel then handles delta < w2.
+template <int D, bool RAW, bool LEFT>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) {
+void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int left) {
     constexpr bool raw = RAW;
+    static_assert(!(RAW && LEFT), "the pre-pass keeps no row copies in LDS");
     using C = KpCfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
@@ -98,10 +106,15 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 
     int pid = blockIdx.x;
     if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    const int bh = pid / nkb, kb = pid - bh * nkb;
+    // (in the pre-pass nkb counts groups of four K' blocks and k0 belongs to the pair)
+    const int bh = pid / nkb, kb = LEFT ? (pid - bh * nkb) * NPAIR + pr : pid - bh * nkb;
     const int b = bh / p.H, h = bh - b * p.H;
     const int k0 = kb * BQ;
-    const int i_hi = (int)((int64_t)k0 + BQ - 1 + w2 < N - 1 ? k0 + BQ - 1 + w2 : N - 1);
+    const int k0_wg = LEFT ? (kb - pr) * BQ : k0;
+    const int k0_end = LEFT ? k0_wg + NPAIR * BQ - 1 : k0 + BQ - 1;               // last K' row of the workgroup
+    const int i_hi = (int)((int64_t)k0_end + w2 < N - 1 ? k0_end + w2 : N - 1);
+    const int nkb_all = (N + BQ - 1) / BQ;
+    if (LEFT && k0_wg + w2 > N - 1) return;          // none of the four blocks has the unit delta = w2
 
     const uint16_t* qp = (const uint16_t*)p.q.p + p.q.off(b, 0, h);
     const uint16_t* k1p = (const uint16_t*)p.k1.p + p.k1.off(b, 0, h);
@@ -110,18 +123,23 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const uint16_t* v2p = (const uint16_t*)p.v2.p + p.v2.off(b, 0, h);
     const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
 
-    const int jt_lo = (k0 - w1 > 0 ? k0 - w1 : 0) / TJ;
+    const int i_lo = LEFT ? k0_wg + w2 : k0;                                      // first query of the workgroup
+    const int jt_lo = (i_lo - w1 > 0 ? i_lo - w1 : 0) / TJ;
     const int jt_hi = i_hi / TJ;
     const int nt = jt_hi - jt_lo + 1;
-    const int n_units = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1;
-    const int nrounds = (n_units + NPAIR - 1) / NPAIR;
+    // the unit delta = w2 exists for this block and the pre-pass took it
+    const bool has_left = left && !LEFT && k0 + w2 <= N - 1;
+    const int n_units = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1 - (has_left ? 1 : 0);
+    const int nrounds = LEFT ? 1 : (n_units + NPAIR - 1) / NPAIR;
     // Tiles a round sweeps: from the first tile of its smallest delta to the last tile of its
     // largest one (tile indices relative to jt_lo).
     auto round_first = [&](int round) {
+        if (LEFT) return 0;
         const int i_min = k0 + round * NPAIR;
         return (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo;
     };
     auto round_last = [&](int round) {
+        if (LEFT) return nt - 1;
         const int dl = (round + 1) * NPAIR - 1 < n_units - 1 ? (round + 1) * NPAIR - 1 : n_units - 1;
         const int i_max = k0 + dl + BQ - 1 < N - 1 ? k0 + dl + BQ - 1 : N - 1;
         return i_max / TJ - jt_lo;
@@ -152,7 +170,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     };
 
     // ---- raw rows, LSE, D and the dQ accumulator -------------------------------------
-    {
+    if constexpr (!LEFT) {
         constexpr int CPR = D / 8;
         for (int c = tid; c < (raw ? RQ * CPR : 0); c += KT) {
             const int row = c / CPR, col = c - row * CPR;
@@ -175,6 +193,16 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             dsum_s[c] = p.dsum[(int64_t)bh * N + r];
         }
         for (int c = tid; c < RQ * C::AS; c += KT) dqacc[c] = 0.f;
+        if (has_left && p.dq.p) {
+            // rows w2 .. w2+31 of the accumulator start from the pre-pass contribution
+            __syncthreads();
+            constexpr int CH = D / 4;
+            const float* src = dq_part + (((int64_t)bh * nkb + kb) * RQ + w2) * D;
+            for (int it = tid; it < BQ * CH; it += KT) {
+                const int row = it / CH, c0 = (it - row * CH) * 4;
+                *(float4*)(dqacc + (w2 + row) * C::AS + c0) = *(const float4*)(src + (int64_t)row * D + c0);
+            }
+        }
     }
 
     // q / dO row of query k0 + rel: the LDS copy or (clamped) global memory
@@ -193,6 +221,16 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             const int r = k0 + rel < N ? k0 + rel : N - 1;
             return dop + (int64_t)r * p.dout.sn;
         }
+    };
+    // K' / V' row k0 + ln of this pair's block
+    const int kc = k0 + ln < N ? k0 + ln : N - 1;
+    auto k2_row = [&]() {
+        if constexpr (LEFT) return k2p + (int64_t)kc * p.k2.sn;
+        else return (const uint16_t*)(k2_s + ln * C::RS);
+    };
+    auto v2_row = [&]() {
+        if constexpr (LEFT) return v2p + (int64_t)kc * p.v2.sn;
+        else return (const uint16_t*)(v2_s + ln * C::RS);
     };
     const float qscale = p.scale * LOG2E;
     const uint32_t smem_addr = lds_address(smem);
@@ -246,12 +284,28 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) pacc[dt][v] = 0.f;
+    // the first pair starts from the pre-pass results (dK' is scaled at the end)
+    auto start_from = [&](const Tensor& t) {
+        if (!(has_left && pr == 0 && t.p)) return;
+        const int tid_i = kp_recompute_here(threadIdx.x);
+        const int k = k0 + (tid_i & 31) < N ? k0 + (tid_i & 31) : N - 1;
+        const uint16_t* src = (const uint16_t*)t.p + t.off(b, k, h) + 4 * ((tid_i >> 5) & 1);
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const uint2 x = *(const uint2*)(src + dt * 32 + 8 * g4);
+                pacc[dt][4 * g4 + 0] = bf16_lo(x.x); pacc[dt][4 * g4 + 1] = bf16_hi(x.x);
+                pacc[dt][4 * g4 + 2] = bf16_lo(x.y); pacc[dt][4 * g4 + 3] = bf16_hi(x.y);
+            }
+    };
 
     if (role == 0) {
         // =============================== P wavefronts ================================
+        start_from(p.dv2);
         for (int round = 0; round < nrounds; ++round) {
-            const int delta = round * NPAIR + pr;
-            const bool ok = delta < n_units;
+            const int delta = LEFT ? w2 : round * NPAIR + pr;
+            const bool ok = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta < n_units;
             const int i = k0 + ln + delta;
             const bool row_ok = i < N;
             const int i_min = k0 + delta;
@@ -268,7 +322,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             float lse2 = 0.f;
             {
                 const uint16_t* qrow = q_row(ln + delta) + hf * 8;
-                const uint16_t* krow = k2_s + ln * C::RS + hf * 8;
+                const uint16_t* krow = k2_row() + hf * 8;
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
                     const uint4 qa = *(const uint4*)(qrow + kk * 16);
@@ -283,7 +337,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     }
                     qf[kk] = r;
                 }
-                if (ok) lse2 = lse_s[ln + delta];
+                if constexpr (LEFT) lse2 = p.lse[(int64_t)bh * N + (i < N ? i : N - 1)] * LOG2E;
+                else if (ok) lse2 = lse_s[ln + delta];
             }
             floatx16 negl;
 #pragma unroll
@@ -352,6 +407,22 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                         pacc[dt][4 * g4 + 3] += racc[dt][4 * g4 + 3] * bf16_hi(x.y);
                     }
             }
+            if constexpr (LEFT) {
+                // pre-pass: dV' of the unit goes to the output tensor as it is
+                if (ok && p.dv2.p && k0 + ln < N) {
+                    uint16_t* dst = (uint16_t*)p.dv2.p + p.dv2.off(b, k0 + ln, h) + 4 * hf;
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int g4 = 0; g4 < 4; ++g4) {
+                            union { __bf16 hh[4]; uint2 u; } o;
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) o.hh[x] = (__bf16)pacc[dt][4 * g4 + x];
+                            *(uint2*)(dst + dt * 32 + 8 * g4) = o.u;
+                        }
+                }
+                return;
+            }
             if (want_dq) {
                 // the dS wavefronts add their dQ contributions in four phases
                 __syncthreads();
@@ -361,9 +432,10 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         }
     } else {
         // =============================== dS wavefronts ===============================
+        start_from(p.dk2);
         for (int round = 0; round < nrounds; ++round) {
-            const int delta = round * NPAIR + pr;
-            const bool ok = delta < n_units;
+            const int delta = LEFT ? w2 : round * NPAIR + pr;
+            const bool ok = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta < n_units;
             const int i_min = k0 + delta;
             const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
             const int sa = ok ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;
@@ -377,7 +449,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             float dsum = 0.f;
             {
                 const uint16_t* drow = do_row(ln + delta) + hf * 8;
-                const uint16_t* vrow = v2_s + ln * C::RS + hf * 8;
+                const uint16_t* vrow = v2_row() + hf * 8;
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
                     const uint4 da = *(const uint4*)(drow + kk * 16);
@@ -392,7 +464,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     }
                     dof[kk] = r;
                 }
-                if (ok) dsum = dsum_s[ln + delta];
+                if constexpr (LEFT) dsum = p.dsum[(int64_t)bh * N + (i_min + ln < N ? i_min + ln : N - 1)];
+                else if (ok) dsum = dsum_s[ln + delta];
             }
             floatx16 dp_prev, negd;
 #pragma unroll
@@ -452,6 +525,42 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                         pacc[dt][4 * g4 + 3] += gacc[dt][4 * g4 + 3] * bf16_hi(x.y);
                     }
             }
+            if constexpr (LEFT) {
+                // pre-pass: dK' of the unit (unscaled) goes to the output tensor, its dQ
+                // contribution G * k2~ (unscaled) to rows w2 .. w2+31 of the block's dQ partial
+                if (ok && k0 + ln < N) {
+                    if (p.dk2.p) {
+                        uint16_t* dst = (uint16_t*)p.dk2.p + p.dk2.off(b, k0 + ln, h) + 4 * hf;
+#pragma unroll
+                        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                            for (int g4 = 0; g4 < 4; ++g4) {
+                                union { __bf16 hh[4]; uint2 u; } o;
+#pragma unroll
+                                for (int x = 0; x < 4; ++x) o.hh[x] = (__bf16)pacc[dt][4 * g4 + x];
+                                *(uint2*)(dst + dt * 32 + 8 * g4) = o.u;
+                            }
+                    }
+                }
+                if (ok && want_dq) {
+                    // (rows of keys past the end of the sequence carry zeros: their G is zero)
+                    float* dst = dq_part + (((int64_t)bh * nkb_all + kb) * RQ + w2 + ln) * D + 4 * hf;
+                    const uint16_t* krow = k2_row() + 4 * hf;
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int g4 = 0; g4 < 4; ++g4) {
+                            const uint2 x = *(const uint2*)(krow + dt * 32 + 8 * g4);
+                            float4 a;
+                            a.x = gacc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.k2_bias);
+                            a.y = gacc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.k2_bias);
+                            a.z = gacc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.k2_bias);
+                            a.w = gacc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.k2_bias);
+                            *(float4*)(dst + dt * 32 + 8 * g4) = a;
+                        }
+                }
+                return;
+            }
             if (want_dq) {
                 // dQ contribution of the unit: dqacc[ln + delta][:] += G * k2~.  The four dS
                 // wavefronts add into the shared fp32 accumulator (scale is applied when the
@@ -465,7 +574,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     const int tid_q = kp_recompute_here(threadIdx.x);
                     const int ln_q = tid_q & 31, hf_q = (tid_q >> 5) & 1;
                     float* arow = dqacc + (ln_q + delta) * C::AS + 4 * hf_q;
-                    const uint16_t* krow = k2_s + ln_q * C::RS + 4 * hf_q;
+                    const uint16_t* krow = k2_s + ln_q * C::RS + 4 * hf_q;      // (main kernel only)
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
                         if (ok) {
@@ -609,11 +718,24 @@ int launch_kp(const Problem& p, hipStream_t st) {
     const bool raw = C::raw_fits(p.w2);
     const size_t lds = C::lds_bytes(p.w2, raw);
     float* part = (float*)p.scratch;
-    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<D, true> : (const void*)mfma_bwd_kp_kernel<D, false>;
+    // one unit left over after the rounds of four: the pre-pass takes it
+    const int left = (p.w2 >= NPAIR && p.w2 % NPAIR == 0) ? 1 : 0;
+    if (left) {
+        const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + C::PX_BYTES;
+        const int ngrp = (nkb + NPAIR - 1) / NPAIR;
+        const int64_t total_left = (int64_t)ngrp * p.B * p.H;
+        if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_left) != hipSuccess)
+            return SA2_ERR_LAUNCH_FAILED;
+        hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, false, true>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
+                           (int)total_left, part, 0);
+        if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    }
+    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<D, true, false> : (const void*)mfma_bwd_kp_kernel<D, false, false>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
-    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, true>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part);
-    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part);
+    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, true, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
+    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, false, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (p.dq.p) {
         const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
