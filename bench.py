@@ -44,9 +44,9 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 380.2e6,                # reads + writes of the forward kernel
-    ("c4", "backward_k_side"): 620.2e6,        # mfma_bwd_kv_kernel
-    ("c4", "backward_kprime_side"): 933.3e6,   # mfma_bwd_kp_kernel 631.8 MB + dq_sum 301.5 MB
+    ("c4", "forward"): 967.0e6,                # pre-pass 522.5 MB + fast kernel 443.4 MB + repair launch 1.1 MB
+    ("c4", "backward_k_side"): 620.9e6,        # mfma_bwd_kv_kernel
+    ("c4", "backward_kprime_side"): 1948.3e6,  # pre-pass 759.6 MB + mfma_bwd_kp_kernel 887.1 MB + dq_sum 301.6 MB
 }
 
 
@@ -193,9 +193,10 @@ def main():
     # recomputation that the pair shares, 2*D*T).
     half_bwd = bwd_flops / 2
     kernels = {
-        "forward": {"kernel": "mfma_fwd_kernel<%d,false> (+ repair launch)" % D, "ms": fwd_ms, "flops": fwd_flops},
+        "forward": {"kernel": "mfma_fwd_kernel<%d> (pre-pass + fast kernel + repair launch)" % D, "ms": fwd_ms,
+                    "flops": fwd_flops},
         "backward_k_side": {"kernel": "mfma_bwd_kv_kernel<%d> (dK, dV)" % D, "ms": bwd_k1_ms, "flops": half_bwd},
-        "backward_kprime_side": {"kernel": "mfma_bwd_kp_kernel<%d> + dq_sum (dQ, dK', dV')" % D, "ms": bwd_rest_ms,
+        "backward_kprime_side": {"kernel": "mfma_bwd_kp_kernel<%d> (pre-pass + main) + dq_sum (dQ, dK', dV')" % D, "ms": bwd_rest_ms,
                                  "flops": half_bwd},
     }
     for k in kernels.values():

@@ -323,10 +323,15 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             {
                 const uint16_t* qrow = q_row(ln + delta) + hf * 8;
                 const uint16_t* krow = k2_row() + hf * 8;
+                uint4 qav[C::DK], kxv[C::DK];       // all reads of the two rows first
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) qav[kk] = *(const uint4*)(qrow + kk * 16);
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) kxv[kk] = *(const uint4*)(krow + kk * 16);
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
-                    const uint4 qa = *(const uint4*)(qrow + kk * 16);
-                    const uint4 kx = *(const uint4*)(krow + kk * 16);
+                    const uint4 qa = qav[kk];
+                    const uint4 kx = kxv[kk];
                     const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
                     const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w};
                     bf16x8 r;
@@ -396,11 +401,14 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             // dV'[k] += R[(k+delta, k)] * dO[k+delta]
             if (ok) {
                 const uint16_t* drow = do_row(ln + delta) + 4 * hf;
+                uint2 dx[4 * C::DT];               // the dO row, read in one batch
+#pragma unroll
+                for (int e = 0; e < 4 * C::DT; ++e) dx[e] = *(const uint2*)(drow + (e >> 2) * 32 + 8 * (e & 3));
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
-                        const uint2 x = *(const uint2*)(drow + dt * 32 + 8 * g4);
+                        const uint2 x = dx[4 * dt + g4];
                         pacc[dt][4 * g4 + 0] += racc[dt][4 * g4 + 0] * bf16_lo(x.x);
                         pacc[dt][4 * g4 + 1] += racc[dt][4 * g4 + 1] * bf16_hi(x.x);
                         pacc[dt][4 * g4 + 2] += racc[dt][4 * g4 + 2] * bf16_lo(x.y);
@@ -450,10 +458,15 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             {
                 const uint16_t* drow = do_row(ln + delta) + hf * 8;
                 const uint16_t* vrow = v2_row() + hf * 8;
+                uint4 dav[C::DK], vxv[C::DK];       // all reads of the two rows first
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) dav[kk] = *(const uint4*)(drow + kk * 16);
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) vxv[kk] = *(const uint4*)(vrow + kk * 16);
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
-                    const uint4 da = *(const uint4*)(drow + kk * 16);
-                    const uint4 vx = *(const uint4*)(vrow + kk * 16);
+                    const uint4 da = dav[kk];
+                    const uint4 vx = vxv[kk];
                     const uint32_t dw[4] = {da.x, da.y, da.z, da.w};
                     const uint32_t vw[4] = {vx.x, vx.y, vx.z, vx.w};
                     bf16x8 r;
@@ -514,11 +527,14 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             // dK'[k] += G[(k+delta, k)] * q[k+delta]   (scale applied at the end)
             if (ok) {
                 const uint16_t* qrow = q_row(ln + delta) + 4 * hf;
+                uint2 qx[4 * C::DT];               // the q row, read in one batch
+#pragma unroll
+                for (int e = 0; e < 4 * C::DT; ++e) qx[e] = *(const uint2*)(qrow + (e >> 2) * 32 + 8 * (e & 3));
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
-                        const uint2 x = *(const uint2*)(qrow + dt * 32 + 8 * g4);
+                        const uint2 x = qx[4 * dt + g4];
                         pacc[dt][4 * g4 + 0] += gacc[dt][4 * g4 + 0] * bf16_lo(x.x);
                         pacc[dt][4 * g4 + 1] += gacc[dt][4 * g4 + 1] * bf16_hi(x.x);
                         pacc[dt][4 * g4 + 2] += gacc[dt][4 * g4 + 2] * bf16_lo(x.y);
@@ -546,11 +562,14 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     // (rows of keys past the end of the sequence carry zeros: their G is zero)
                     float* dst = dq_part + (((int64_t)bh * nkb_all + kb) * RQ + w2 + ln) * D + 4 * hf;
                     const uint16_t* krow = k2_row() + 4 * hf;
+                    uint2 kx[4 * C::DT];           // the K' row, read in one batch
+#pragma unroll
+                    for (int e = 0; e < 4 * C::DT; ++e) kx[e] = *(const uint2*)(krow + (e >> 2) * 32 + 8 * (e & 3));
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int g4 = 0; g4 < 4; ++g4) {
-                            const uint2 x = *(const uint2*)(krow + dt * 32 + 8 * g4);
+                            const uint2 x = kx[4 * dt + g4];
                             float4 a;
                             a.x = gacc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.k2_bias);
                             a.y = gacc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.k2_bias);

@@ -319,12 +319,18 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 const uint16_t* qrow;
                 if constexpr (LEFT) qrow = qp + (int64_t)ic * p.q.sn + hf * 8;
                 else qrow = q_s + ln * C::KS + hf * 8;
+                // (all reads of the two rows first: from global memory they overlap)
+                uint4 qav[C::DK], kbv[C::DK];
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) kbv[kk] = *(const uint4*)(krow + kk * 16);
+#pragma unroll
+                for (int kk = 0; kk < C::DK; ++kk) qav[kk] = *(const uint4*)(qrow + kk * 16);
                 auto form_q = [&](auto BIASED) {
                     const float kbias = decltype(BIASED)::value ? p.k2_bias : 0.f;
 #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) {
-                        const uint4 qa = *(const uint4*)(qrow + kk * 16);
-                        const uint4 kb = *(const uint4*)(krow + kk * 16);
+                        const uint4 qa = qav[kk];
+                        const uint4 kb = kbv[kk];
                         const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
                         const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
                         bf16x8 r;
@@ -570,11 +576,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 const int kr = i - delta > 0 ? i - delta : 0;
                 const uint16_t* vrow = v2p + (int64_t)kr * p.v2.sn + 4 * hf;
                 uint16_t* orow = (uint16_t*)p.out.p + p.out.off(b, i, h) + 4 * hf;
+                uint2 vx[4 * C::DT];               // the V' row, read in one batch
+#pragma unroll
+                for (int e = 0; e < 4 * C::DT; ++e) vx[e] = *(const uint2*)(vrow + (e >> 2) * 32 + 8 * (e & 3));
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
-                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        const uint2 x = vx[4 * dt + g4];
                         union { __bf16 h[4]; uint2 u; } o;
                         o.h[0] = (__bf16)(inv * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
                         o.h[1] = (__bf16)(inv * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
@@ -596,6 +605,18 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
         const int tid_m = recompute_here(threadIdx.x);
         const int ln_m = tid_m & 31, hf_m = (tid_m >> 5) & 1;
         const int aq = tid_m >> 4, ac = (tid_m & 15) * ACN;
+        // the V' row of this lane's query, read in one batch before the exchange below
+        const uint16_t* vrow;
+        if constexpr (SIDE) {
+            vrow = v2_s + (ok ? ln_m + w2 - delta : 0) * C::KS + 4 * hf_m;
+        } else {
+            const int iq = i0 + ln_m < N ? i0 + ln_m : N - 1;
+            const int vr = ok && iq - delta > 0 ? iq - delta : 0;
+            vrow = v2p + (int64_t)vr * p.v2.sn + 4 * hf_m;
+        }
+        uint2 vx[4 * C::DT];
+#pragma unroll
+        for (int e = 0; e < 4 * C::DT; ++e) vx[e] = *(const uint2*)(vrow + (e >> 2) * 32 + 8 * (e & 3));
         const float lt = l + other_half(l);
         if (hf_m == 0) {
             xch_m[wave * BQ + ln_m] = m;
@@ -624,14 +645,6 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
         // other four use the two stage buffers that hold no tile of the next round.  Then
         // every thread adds its slice of the seven slabs in wavefront order.
         const float cw = ok ? fast_exp2(m - Muse) : 0.f;
-        const uint16_t* vrow;
-        if constexpr (SIDE) {
-            vrow = v2_s + (ok ? ln_m + w2 - delta : 0) * C::KS + 4 * hf_m;
-        } else {
-            const int iq = i0 + ln_m < N ? i0 + ln_m : N - 1;
-            const int vr = ok && iq - delta > 0 ? iq - delta : 0;
-            vrow = v2p + (int64_t)vr * p.v2.sn + 4 * hf_m;
-        }
         auto slab_of = [&](int w) -> uint16_t* {
             if (w < 4) return slabs + (w - 1) * (BQ * C::SS);
             const int fb = (buf + 2 + ((w - 4) >> 1)) & (C::NSTAGE - 1);      // the two stages after the next round's first two
@@ -648,7 +661,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
-                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        const uint2 x = vx[4 * dt + g4];
                         float4 o = *(float4*)(arow + dt * 32 + 8 * g4);
                         if (PLAIN) {
                             o.x += racc[dt][4 * g4 + 0] * bf16_lo(x.x);
@@ -670,7 +683,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
-                        const uint2 x = *(const uint2*)(vrow + dt * 32 + 8 * g4);
+                        const uint2 x = vx[4 * dt + g4];
                         union { __bf16 h[4]; uint2 u; } o;
                         if (PLAIN) {
                             o.h[0] = (__bf16)(racc[dt][4 * g4 + 0] * bf16_lo(x.x));
