@@ -110,7 +110,7 @@ int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, c
     hipStream_t st = (hipStream_t)hip_stream;
     const bool mfma = pick_mfma(p, dtype, flags, false, &rc);
     if (rc != SA2_OK) return rc;
-    return mfma ? launch_mfma_fwd(p, st) : launch_generic_fwd(p, dtype, st);
+    return mfma ? launch_mfma_fwd(p, dtype, st) : launch_generic_fwd(p, dtype, st);
 }
 
 size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int dtype, unsigned flags) {
@@ -166,7 +166,7 @@ int sa2_backward(const void* q, const void* k1, const void* k2, const void* v1, 
     hipStream_t st = (hipStream_t)hip_stream;
     const bool mfma = pick_mfma(p, dtype, flags, true, &rc);
     if (rc != SA2_OK) return rc;
-    return mfma ? launch_mfma_bwd(p, st) : launch_generic_bwd(p, dtype, st);
+    return mfma ? launch_mfma_bwd(p, dtype, st) : launch_generic_bwd(p, dtype, st);
 }
 
 int sa2_rowdot(const void* out, const void* dout, float* dsum, int B, int N, int H, int D,

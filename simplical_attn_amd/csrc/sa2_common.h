@@ -75,15 +75,15 @@ size_t generic_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 bool mfma_supported(int B, int N, int H, int D, int w1, int w2, int dtype);
 bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype);
 bool mfma_layout_ok(const Problem& p, bool backward);
-int launch_mfma_fwd(const Problem& p, hipStream_t st);
-int launch_mfma_bwd(const Problem& p, hipStream_t st);
+int launch_mfma_fwd(const Problem& p, int dtype, hipStream_t st);
+int launch_mfma_bwd(const Problem& p, int dtype, hipStream_t st);
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 // K'-side backward kernel (dQ, dK', dV') that keeps its partial sums on chip
 bool kp_fits(int D, int w2);
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2);
-int launch_mfma_bwd_kp(const Problem& p, hipStream_t st);
+int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st);
 // K-side backward kernel (dK, dV) with paired wavefronts
 bool kv_fits(int D, int w2);
-int launch_mfma_bwd_kv(const Problem& p, hipStream_t st);
+int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st);
 
 }  // namespace sa2

@@ -616,7 +616,9 @@ int launch_row_part(const Problem& p, hipStream_t st) {
 }  // namespace
 
 bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
-    return mfma_supported(B, N, H, D, w1, w2, dtype);
+    if (!mfma_supported(B, N, H, D, w1, w2, dtype)) return false;
+    // the workspace fallback kernels for wide K' windows exist for bf16 only
+    return dtype == SA2_BF16 || (kp_fits(D, w2) && kv_fits(D, w2));
 }
 
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
@@ -626,16 +628,16 @@ size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
     return 2 * one;
 }
 
-int launch_mfma_bwd(const Problem& p, hipStream_t st) {
-    int rc = launch_rowdot(p.out, p.dout, p.dsum, p.B, p.N, p.H, p.D, SA2_BF16, st);
+int launch_mfma_bwd(const Problem& p, int dtype, hipStream_t st) {
+    int rc = launch_rowdot(p.out, p.dout, p.dsum, p.B, p.N, p.H, p.D, dtype, st);
     if (rc != SA2_OK) return rc;
     if (p.dq.p || p.dk2.p || p.dv2.p) {
-        if (kp_fits(p.D, p.w2)) rc = launch_mfma_bwd_kp(p, st);
+        if (kp_fits(p.D, p.w2)) rc = launch_mfma_bwd_kp(p, dtype, st);
         else rc = p.D == 128 ? launch_row_part<128>(p, st) : launch_row_part<64>(p, st);
         if (rc != SA2_OK) return rc;
     }
     if (p.dk1.p || p.dv1.p) {
-        if (kv_fits(p.D, p.w2)) rc = launch_mfma_bwd_kv(p, st);
+        if (kv_fits(p.D, p.w2)) rc = launch_mfma_bwd_kv(p, dtype, st);
         else rc = p.D == 128 ? launch_col_part<128>(p, st) : launch_col_part<64>(p, st);
     }
     return rc;

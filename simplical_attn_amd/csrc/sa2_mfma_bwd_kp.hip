@@ -1,4 +1,4 @@
-// bf16 MFMA backward for gfx950, the K'-side kernel: dQ, dK' and dV'.
+// MFMA backward for gfx950 (bf16 or fp16 elements), the K'-side kernel: dQ, dK' and dV'.
 //
 // Expanded rows r = (i, k), k = i - delta in the K' window of i.  A workgroup owns 32
 // consecutive K' rows k0..k0+31 and every delta: unit delta is the 32 rows
@@ -16,7 +16,7 @@
 //
 // Eight wavefronts, two per SIMD, form four pairs that each hold one unit per round and
 // sweep the K1/V1 window in 32-key tiles staged through a three-deep LDS ring:
-//   the "P" wavefront computes S^T = K1.Q~^T, P = exp2(S - LSE), hands P (bf16) to its
+//   the "P" wavefront computes S^T = K1.Q~^T, P = exp2(S - LSE), hands P (16 bit) to its
 //       partner through LDS and accumulates R^T += V1^T.P^T;
 //   the "dS" wavefront computes dP^T = V1.dO~^T and, one tile behind, dS = P*(dP - D) and
 //       G^T += K1^T.dS^T.
@@ -77,11 +77,13 @@ struct KpCfg {
 // four (w2 + 1 = 4n + 1).  A workgroup takes four consecutive K' blocks, one per wavefront
 // pair, and computes the unit delta = w2 of each in one shared sweep of K/V tiles.  Its
 // results go where the main kernel (launched next with left = 1) picks them up: dK'
-// (unscaled) and dV' as bf16 in the output tensors, the dQ contribution as fp32 in rows
+// (unscaled) and dV' in the element type in the output tensors, the dQ contribution as fp32 in rows
 // w2 .. w2+31 of the block's dQ partial.  The main kernel then handles delta < w2.
-template <int D, bool RAW, bool LEFT>
+template <class E, int D, bool RAW, bool LEFT>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int left) {
+    typedef typename E::scalar EL;
+    typedef typename E::x8 X8;
     constexpr bool raw = RAW;
     static_assert(!(RAW && LEFT), "the pre-pass keeps no row copies in LDS");
     using C = KpCfg<D>;
@@ -295,8 +297,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const uint2 x = *(const uint2*)(src + dt * 32 + 8 * g4);
-                pacc[dt][4 * g4 + 0] = bf16_lo(x.x); pacc[dt][4 * g4 + 1] = bf16_hi(x.x);
-                pacc[dt][4 * g4 + 2] = bf16_lo(x.y); pacc[dt][4 * g4 + 3] = bf16_hi(x.y);
+                pacc[dt][4 * g4 + 0] = E::lo(x.x); pacc[dt][4 * g4 + 1] = E::hi(x.x);
+                pacc[dt][4 * g4 + 2] = E::lo(x.y); pacc[dt][4 * g4 + 3] = E::hi(x.y);
             }
     };
 
@@ -318,7 +320,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) racc[dt][v] = 0.f;
-            bf16x8 qf[C::DK];
+            X8 qf[C::DK];
             float lse2 = 0.f;
             {
                 const uint16_t* qrow = q_row(ln + delta) + hf * 8;
@@ -334,11 +336,11 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     const uint4 kx = kxv[kk];
                     const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
                     const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w};
-                    bf16x8 r;
+                    X8 r;
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
-                        r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
+                        r[2 * t] = (EL)(E::lo(qw[t]) * (E::lo(kw[t]) + p.k2_bias) * qscale);
+                        r[2 * t + 1] = (EL)(E::hi(qw[t]) * (E::hi(kw[t]) + p.k2_bias) * qscale);
                     }
                     qf[kk] = r;
                 }
@@ -354,13 +356,13 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 if (s >= sa && s <= sb) {
                     const int j0 = (jt_lo + s) * TJ;
                     const uint32_t ks_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u;
-                    bf16x8 ka[C::DK];
+                    X8 ka[C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + row_lane + kk * KKB);
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_x8<X8>(ks_addr + row_lane + kk * KKB);
                     floatx16 sh;
                     const bool plain = rows_full && j0 + TJ - 1 <= i_min && j0 >= i_max - w1;
                     if (__builtin_expect(plain, 1)) {
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], negl, 0, 0, 0);
+                        sh = E::mfma(ka[0], qf[0], negl, 0, 0, 0);
                     } else {
                         asm volatile("" ::: "memory");
                         // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
@@ -371,16 +373,16 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                             const int c = 8 * (v >> 2) + (v & 3);
                             ct[v] = (row_ok & (c <= hi) & (c >= lo)) ? negl[0] : -INFINITY;
                         }
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], ct, 0, 0, 0);
+                        sh = E::mfma(ka[0], qf[0], ct, 0, 0, 0);
                     }
 #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sh, 0, 0, 0);
-                    bf16x8 pb[2];
+                        sh = E::mfma(ka[kk], qf[kk], sh, 0, 0, 0);
+                    X8 pb[2];
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                        for (int t = 0; t < 8; ++t) pb[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t]);
+                        for (int t = 0; t < 8; ++t) pb[ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
                     lds_half_operand vh[4 * C::DT];
                     issue_tr(ks_addr + (uint32_t)C::TILE_BYTES + col_lane, vh);
                     {
@@ -393,7 +395,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks)
-                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_join(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]),
+                            racc[dt] = E::mfma(lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]),
                                                                                pb[ks], racc[dt], 0, 0, 0);
                 }
                 advance();
@@ -409,10 +411,10 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
                         const uint2 x = dx[4 * dt + g4];
-                        pacc[dt][4 * g4 + 0] += racc[dt][4 * g4 + 0] * bf16_lo(x.x);
-                        pacc[dt][4 * g4 + 1] += racc[dt][4 * g4 + 1] * bf16_hi(x.x);
-                        pacc[dt][4 * g4 + 2] += racc[dt][4 * g4 + 2] * bf16_lo(x.y);
-                        pacc[dt][4 * g4 + 3] += racc[dt][4 * g4 + 3] * bf16_hi(x.y);
+                        pacc[dt][4 * g4 + 0] += racc[dt][4 * g4 + 0] * E::lo(x.x);
+                        pacc[dt][4 * g4 + 1] += racc[dt][4 * g4 + 1] * E::hi(x.x);
+                        pacc[dt][4 * g4 + 2] += racc[dt][4 * g4 + 2] * E::lo(x.y);
+                        pacc[dt][4 * g4 + 3] += racc[dt][4 * g4 + 3] * E::hi(x.y);
                     }
             }
             if constexpr (LEFT) {
@@ -423,9 +425,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int g4 = 0; g4 < 4; ++g4) {
-                            union { __bf16 hh[4]; uint2 u; } o;
+                            union { EL hh[4]; uint2 u; } o;
 #pragma unroll
-                            for (int x = 0; x < 4; ++x) o.hh[x] = (__bf16)pacc[dt][4 * g4 + x];
+                            for (int x = 0; x < 4; ++x) o.hh[x] = (EL)pacc[dt][4 * g4 + x];
                             *(uint2*)(dst + dt * 32 + 8 * g4) = o.u;
                         }
                 }
@@ -453,7 +455,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) gacc[dt][v] = 0.f;
-            bf16x8 dof[C::DK];
+            X8 dof[C::DK];
             float dsum = 0.f;
             {
                 const uint16_t* drow = do_row(ln + delta) + hf * 8;
@@ -469,11 +471,11 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     const uint4 vx = vxv[kk];
                     const uint32_t dw[4] = {da.x, da.y, da.z, da.w};
                     const uint32_t vw[4] = {vx.x, vx.y, vx.z, vx.w};
-                    bf16x8 r;
+                    X8 r;
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        r[2 * t] = (__bf16)(bf16_lo(dw[t]) * (bf16_lo(vw[t]) + p.v2_bias));
-                        r[2 * t + 1] = (__bf16)(bf16_hi(dw[t]) * (bf16_hi(vw[t]) + p.v2_bias));
+                        r[2 * t] = (EL)(E::lo(dw[t]) * (E::lo(vw[t]) + p.v2_bias));
+                        r[2 * t + 1] = (EL)(E::hi(dw[t]) * (E::hi(vw[t]) + p.v2_bias));
                     }
                     dof[kk] = r;
                 }
@@ -485,24 +487,24 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             for (int v = 0; v < 16; ++v) { dp_prev[v] = 0.f; negd[v] = -dsum; }
             // dS of the tile handled in the previous step and its G MFMAs
             auto consume = [&]() {
-                typedef const bf16x8 __attribute__((address_space(3)))* lds_b8;
+                typedef const X8 __attribute__((address_space(3)))* lds_b8;
                 const uint32_t a = px_addr + (uint32_t)(((g - 1) & 1) * 64 * 32);
-                const bf16x8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
+                const X8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
                 const int pb = buf == 0 ? C::NSTAGE - 1 : buf - 1;
                 lds_half_operand kh[4 * C::DT];
                 issue_tr(smem_addr + (uint32_t)(pb * C::STAGE) * 2u + col_lane, kh);
                 lds_settle(kh);
-                bf16x8 dsb[2];
+                X8 dsb[2];
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    dsb[0][t] = (__bf16)((float)p0[t] * dp_prev[t]);
-                    dsb[1][t] = (__bf16)((float)p1[t] * dp_prev[8 + t]);
+                    dsb[0][t] = (EL)((float)p0[t] * dp_prev[t]);
+                    dsb[1][t] = (EL)((float)p1[t] * dp_prev[8 + t]);
                 }
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
-                        gacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_join(kh[4 * dt + 2 * ks], kh[4 * dt + 2 * ks + 1]),
+                        gacc[dt] = E::mfma(lds_join<X8>(kh[4 * dt + 2 * ks], kh[4 * dt + 2 * ks + 1]),
                                                                            dsb[ks], gacc[dt], 0, 0, 0);
             };
             const int s_end = round_last(round);
@@ -511,13 +513,13 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 if (s - 1 >= sa && s - 1 <= sb) consume();
                 if (s >= sa && s <= sb) {
                     const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u + (uint32_t)C::TILE_BYTES;
-                    bf16x8 va[C::DK];
+                    X8 va[C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) va[kk] = lds_read_bf16x8(vs_addr + row_lane + kk * KKB);
-                    dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[0], dof[0], negd, 0, 0, 0);
+                    for (int kk = 0; kk < C::DK; ++kk) va[kk] = lds_read_x8<X8>(vs_addr + row_lane + kk * KKB);
+                    dp_prev = E::mfma(va[0], dof[0], negd, 0, 0, 0);
 #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)
-                        dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[kk], dof[kk], dp_prev, 0, 0, 0);
+                        dp_prev = E::mfma(va[kk], dof[kk], dp_prev, 0, 0, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
                 }
@@ -535,10 +537,10 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
                         const uint2 x = qx[4 * dt + g4];
-                        pacc[dt][4 * g4 + 0] += gacc[dt][4 * g4 + 0] * bf16_lo(x.x);
-                        pacc[dt][4 * g4 + 1] += gacc[dt][4 * g4 + 1] * bf16_hi(x.x);
-                        pacc[dt][4 * g4 + 2] += gacc[dt][4 * g4 + 2] * bf16_lo(x.y);
-                        pacc[dt][4 * g4 + 3] += gacc[dt][4 * g4 + 3] * bf16_hi(x.y);
+                        pacc[dt][4 * g4 + 0] += gacc[dt][4 * g4 + 0] * E::lo(x.x);
+                        pacc[dt][4 * g4 + 1] += gacc[dt][4 * g4 + 1] * E::hi(x.x);
+                        pacc[dt][4 * g4 + 2] += gacc[dt][4 * g4 + 2] * E::lo(x.y);
+                        pacc[dt][4 * g4 + 3] += gacc[dt][4 * g4 + 3] * E::hi(x.y);
                     }
             }
             if constexpr (LEFT) {
@@ -551,9 +553,9 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                         for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                             for (int g4 = 0; g4 < 4; ++g4) {
-                                union { __bf16 hh[4]; uint2 u; } o;
+                                union { EL hh[4]; uint2 u; } o;
 #pragma unroll
-                                for (int x = 0; x < 4; ++x) o.hh[x] = (__bf16)pacc[dt][4 * g4 + x];
+                                for (int x = 0; x < 4; ++x) o.hh[x] = (EL)pacc[dt][4 * g4 + x];
                                 *(uint2*)(dst + dt * 32 + 8 * g4) = o.u;
                             }
                     }
@@ -571,10 +573,10 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                         for (int g4 = 0; g4 < 4; ++g4) {
                             const uint2 x = kx[4 * dt + g4];
                             float4 a;
-                            a.x = gacc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.k2_bias);
-                            a.y = gacc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.k2_bias);
-                            a.z = gacc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.k2_bias);
-                            a.w = gacc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.k2_bias);
+                            a.x = gacc[dt][4 * g4 + 0] * (E::lo(x.x) + p.k2_bias);
+                            a.y = gacc[dt][4 * g4 + 1] * (E::hi(x.x) + p.k2_bias);
+                            a.z = gacc[dt][4 * g4 + 2] * (E::lo(x.y) + p.k2_bias);
+                            a.w = gacc[dt][4 * g4 + 3] * (E::hi(x.y) + p.k2_bias);
                             *(float4*)(dst + dt * 32 + 8 * g4) = a;
                         }
                 }
@@ -613,10 +615,10 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                                 const int sb16 = ((P0 + t) & 3) + 4 * (e >> 1);
                                 const int dt = sb16 >> 1, g4 = 2 * (sb16 & 1) + (e & 1);
                                 const float kb = WITH_BIAS ? p.k2_bias : 0.f;
-                                a[e].x += gacc[dt][4 * g4 + 0] * (bf16_lo(x[e].x) + kb);
-                                a[e].y += gacc[dt][4 * g4 + 1] * (bf16_hi(x[e].x) + kb);
-                                a[e].z += gacc[dt][4 * g4 + 2] * (bf16_lo(x[e].y) + kb);
-                                a[e].w += gacc[dt][4 * g4 + 3] * (bf16_hi(x[e].y) + kb);
+                                a[e].x += gacc[dt][4 * g4 + 0] * (E::lo(x[e].x) + kb);
+                                a[e].y += gacc[dt][4 * g4 + 1] * (E::hi(x[e].x) + kb);
+                                a[e].z += gacc[dt][4 * g4 + 2] * (E::lo(x[e].y) + kb);
+                                a[e].w += gacc[dt][4 * g4 + 3] * (E::hi(x[e].y) + kb);
                                 *(float4*)(arow + (sb16 >> 1) * 32 + 8 * g4) = a[e];
                             }
                         }
@@ -688,18 +690,19 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
             }
             const float sc = which ? p.scale : 1.f;
-            union { __bf16 hh[8]; uint4 u; } o;
+            union { EL hh[8]; uint4 u; } o;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) o.hh[c] = (__bf16)(acc[c] * sc);
+            for (int c = 0; c < 8; ++c) o.hh[c] = (EL)(acc[c] * sc);
             *(uint4*)((uint16_t*)t.p + t.off(b, k, h) + c0) = o.u;
         }
     }
 }
 
 // dQ[i] = sum of the partials of the K' blocks that reach query i, in block order.
-template <int D>
+template <class E, int D>
 __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const float* __restrict__ dq_part, int nkb,
                                                              int64_t items) {
+    typedef typename E::scalar EL;
     constexpr int CH = D / 8;
     const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (it >= items) return;
@@ -721,13 +724,13 @@ __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const f
         acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
         acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
     }
-    union { __bf16 hh[8]; uint4 u; } o;
+    union { EL hh[8]; uint4 u; } o;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) o.hh[c] = (__bf16)acc[c];
+    for (int c = 0; c < 8; ++c) o.hh[c] = (EL)acc[c];
     *(uint4*)((uint16_t*)p.dq.p + p.dq.off(b, i, h) + c0) = o.u;
 }
 
-template <int D>
+template <class E, int D>
 int launch_kp(const Problem& p, hipStream_t st) {
     using C = KpCfg<D>;
     const int nkb = (p.N + BQ - 1) / BQ;
@@ -743,22 +746,22 @@ int launch_kp(const Problem& p, hipStream_t st) {
         const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + C::PX_BYTES;
         const int ngrp = (nkb + NPAIR - 1) / NPAIR;
         const int64_t total_left = (int64_t)ngrp * p.B * p.H;
-        if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<E, D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)lds_left) != hipSuccess)
             return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, false, true>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
+        hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, true>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
                            (int)total_left, part, 0);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
-    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<D, true, false> : (const void*)mfma_bwd_kp_kernel<D, false, false>;
+    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<E, D, true, false> : (const void*)mfma_bwd_kp_kernel<E, D, false, false>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
-    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, true, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
-    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<D, false, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
+    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, true, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
+    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (p.dq.p) {
         const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
-        hipLaunchKernelGGL(mfma_bwd_dq_sum_kernel<D>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p, part,
+        hipLaunchKernelGGL((mfma_bwd_dq_sum_kernel<E, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p, part,
                            nkb, items);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
@@ -774,8 +777,9 @@ size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {
     return (size_t)B * H * nkb * (size_t)(BQ + w2) * D * sizeof(float);
 }
 
-int launch_mfma_bwd_kp(const Problem& p, hipStream_t st) {
-    return p.D == 128 ? launch_kp<128>(p, st) : launch_kp<64>(p, st);
+int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st) {
+    if (dtype == SA2_F16) return p.D == 128 ? launch_kp<ElemF16, 128>(p, st) : launch_kp<ElemF16, 64>(p, st);
+    return p.D == 128 ? launch_kp<ElemBF16, 128>(p, st) : launch_kp<ElemBF16, 64>(p, st);
 }
 
 }  // namespace sa2

@@ -1,11 +1,11 @@
-// bf16 MFMA backward for gfx950, the K-side kernel: dK and dV.
+// MFMA backward for gfx950 (bf16 or fp16 elements), the K-side kernel: dK and dV.
 //
 // A workgroup owns 128 consecutive K/V rows, 32 per wavefront pair, resident in registers
 // as MFMA B operands.  It streams every unit of expanded rows that can see them: unit
 // (query block ib, delta) is the 32 rows r = (i0 + r, k = i - delta) with
 // Q~[r] = q[i] * k2~[k] * scale*log2(e) and dO~[r] = dO[i] * v2~[k], formed by the whole
 // workgroup into a three-deep LDS ring one step ahead of their use.  Per unit and pair:
-//   the "P" wavefront computes S = Q~.K^T - LSE, P = exp2(S), hands P (bf16) to its partner
+//   the "P" wavefront computes S = Q~.K^T - LSE, P = exp2(S), hands P (16 bit) to its partner
 //       through LDS and accumulates dV^T += dO~^T.P;
 //   the "dS" wavefront computes dP = dO~.V^T - D and, one unit behind, dS = P*dP and
 //       dK^T += Q~^T.dS.
@@ -42,9 +42,11 @@ struct KvCfg {
 };
 
 // BIAS = false: k2_bias and v2_bias are both zero (the reference's default), the adds drop out.
-template <int D, bool BIAS>
+template <class E, int D, bool BIAS>
 __global__ __launch_bounds__(VT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
+    typedef typename E::scalar EL;
+    typedef typename E::x8 X8;
     using C = KvCfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
@@ -78,12 +80,12 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
 
     // K rows (P wavefront) or V rows (dS wavefront) of the pair as the resident B operand
-    bf16x8 kvf[C::DK];
+    X8 kvf[C::DK];
     {
         const Tensor& t = role ? p.v1 : p.k1;
         const uint16_t* src = (const uint16_t*)t.p + t.off(b, jc, h) + hf * 8;
 #pragma unroll
-        for (int kk = 0; kk < C::DK; ++kk) kvf[kk] = *(const bf16x8*)(src + kk * 16);
+        for (int kk = 0; kk < C::DK; ++kk) kvf[kk] = *(const X8*)(src + kk * 16);
     }
     floatx16 oacc[C::DT];                        // dV^T (P wavefront) or dK^T (dS wavefront)
 #pragma unroll
@@ -112,10 +114,10 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             const uint4 da = *(const uint4*)(dop + (int64_t)i * p.dout.sn + col * 8);
             float* qd = q_s + row * C::FS + col * 8;
             float* dd = do_s + row * C::FS + col * 8;
-            *(float4*)qd = make_float4(bf16_lo(qa.x) * qscale, bf16_hi(qa.x) * qscale, bf16_lo(qa.y) * qscale, bf16_hi(qa.y) * qscale);
-            *(float4*)(qd + 4) = make_float4(bf16_lo(qa.z) * qscale, bf16_hi(qa.z) * qscale, bf16_lo(qa.w) * qscale, bf16_hi(qa.w) * qscale);
-            *(float4*)dd = make_float4(bf16_lo(da.x), bf16_hi(da.x), bf16_lo(da.y), bf16_hi(da.y));
-            *(float4*)(dd + 4) = make_float4(bf16_lo(da.z), bf16_hi(da.z), bf16_lo(da.w), bf16_hi(da.w));
+            *(float4*)qd = make_float4(E::lo(qa.x) * qscale, E::hi(qa.x) * qscale, E::lo(qa.y) * qscale, E::hi(qa.y) * qscale);
+            *(float4*)(qd + 4) = make_float4(E::lo(qa.z) * qscale, E::hi(qa.z) * qscale, E::lo(qa.w) * qscale, E::hi(qa.w) * qscale);
+            *(float4*)dd = make_float4(E::lo(da.x), E::hi(da.x), E::lo(da.y), E::hi(da.y));
+            *(float4*)(dd + 4) = make_float4(E::lo(da.z), E::hi(da.z), E::lo(da.w), E::hi(da.w));
         }
         for (int c = tid; c < SR * CPR; c += VT) {
             const int row = c / CPR, col = c - row * CPR;
@@ -154,24 +156,24 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
         const uint4 vx = *(const uint4*)(v2_s + kr * C::RS + col * 8);
         const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w}, vw[4] = {vx.x, vx.y, vx.z, vx.w};
         const float kb = BIAS ? p.k2_bias : 0.f, vb = BIAS ? p.v2_bias : 0.f;
-        bf16x8 r, d;
+        X8 r, d;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             if (BIAS) {
-                r[2 * t] = (__bf16)(qv[2 * t] * (bf16_lo(kw[t]) + kb));
-                r[2 * t + 1] = (__bf16)(qv[2 * t + 1] * (bf16_hi(kw[t]) + kb));
-                d[2 * t] = (__bf16)(dv[2 * t] * (bf16_lo(vw[t]) + vb));
-                d[2 * t + 1] = (__bf16)(dv[2 * t + 1] * (bf16_hi(vw[t]) + vb));
+                r[2 * t] = (EL)(qv[2 * t] * (E::lo(kw[t]) + kb));
+                r[2 * t + 1] = (EL)(qv[2 * t + 1] * (E::hi(kw[t]) + kb));
+                d[2 * t] = (EL)(dv[2 * t] * (E::lo(vw[t]) + vb));
+                d[2 * t + 1] = (EL)(dv[2 * t + 1] * (E::hi(vw[t]) + vb));
             } else {
-                r[2 * t] = (__bf16)(qv[2 * t] * bf16_lo(kw[t]));
-                r[2 * t + 1] = (__bf16)(qv[2 * t + 1] * bf16_hi(kw[t]));
-                d[2 * t] = (__bf16)(dv[2 * t] * bf16_lo(vw[t]));
-                d[2 * t + 1] = (__bf16)(dv[2 * t + 1] * bf16_hi(vw[t]));
+                r[2 * t] = (EL)(qv[2 * t] * E::lo(kw[t]));
+                r[2 * t + 1] = (EL)(qv[2 * t + 1] * E::hi(kw[t]));
+                d[2 * t] = (EL)(dv[2 * t] * E::lo(vw[t]));
+                d[2 * t + 1] = (EL)(dv[2 * t + 1] * E::hi(vw[t]));
             }
         }
         uint16_t* dst = units + slot * C::UNIT + row * C::TS + col * 8;
-        *(bf16x8*)dst = r;
-        *(bf16x8*)(dst + C::TILE) = d;
+        *(X8*)dst = r;
+        *(X8*)(dst + C::TILE) = d;
     };
 
     const uint32_t units_addr = lds_address(units);
@@ -202,26 +204,26 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
 
         // dS of the previous unit and its dK MFMAs (dS wavefronts)
         auto consume = [&](int pslot, int pstep) {
-            typedef const bf16x8 __attribute__((address_space(3)))* lds_b8;
+            typedef const X8 __attribute__((address_space(3)))* lds_b8;
             const uint32_t a = px_addr + (uint32_t)((pstep & 1) * 64 * 32);
-            const bf16x8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
+            const X8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
             const uint32_t qt_addr = units_addr + (uint32_t)(pslot * C::UNIT) * 2u + col_lane;
-            bf16x8 qt[C::DT][2];
+            X8 qt[C::DT][2];
     #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) qt[dt][ks] = lds_column_operand_at<C::TS>(qt_addr + dt * 64, ks);
-            bf16x8 dsb[2];
+                for (int ks = 0; ks < 2; ++ks) qt[dt][ks] = lds_column_operand_at<C::TS, X8>(qt_addr + dt * 64, ks);
+            X8 dsb[2];
     #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                dsb[0][t] = (__bf16)((float)p0[t] * dp_prev[t]);
-                dsb[1][t] = (__bf16)((float)p1[t] * dp_prev[8 + t]);
+                dsb[0][t] = (EL)((float)p0[t] * dp_prev[t]);
+                dsb[1][t] = (EL)((float)p1[t] * dp_prev[8 + t]);
             }
     #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qt[dt][ks], dsb[ks], oacc[dt], 0, 0, 0);
+                    oacc[dt] = E::mfma(qt[dt][ks], dsb[ks], oacc[dt], 0, 0, 0);
         };
 
         while (true) {
@@ -240,14 +242,14 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             const uint32_t u_addr = units_addr + (uint32_t)(slot * C::UNIT) * 2u;
             if (ROLE == 0) {
                 if (act) {
-                    bf16x8 qa[C::DK];
+                    X8 qa[C::DK];
     #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) qa[kk] = lds_read_bf16x8(u_addr + row_lane + kk * 32);
+                    for (int kk = 0; kk < C::DK; ++kk) qa[kk] = lds_read_x8<X8>(u_addr + row_lane + kk * 32);
                     floatx16 sh;
                     const bool interior = (i0 >= jw + 31) && ((int64_t)i0 + 31 <= (int64_t)jw + w1) && (i0 + BQ - 1 < N) &&
                                           (i0 >= delta);
                     if (__builtin_expect(interior, 1)) {
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[0], kvf[0], negr, 0, 0, 0);
+                        sh = E::mfma(qa[0], kvf[0], negr, 0, 0, 0);
                     } else {
                         asm volatile("" ::: "memory");
                         // element v of this lane is query i0 + 8*(v/4) + 4*hf + v%4, column j
@@ -260,46 +262,46 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                             const int c = 8 * (v >> 2) + (v & 3);
                             ct[v] = ((j < N) & (c >= lo) & (c <= hi) & (c >= dlo) & (c <= nhi)) ? negr[v] : -INFINITY;
                         }
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[0], kvf[0], ct, 0, 0, 0);
+                        sh = E::mfma(qa[0], kvf[0], ct, 0, 0, 0);
                     }
     #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)
-                        sh = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[kk], kvf[kk], sh, 0, 0, 0);
-                    bf16x8 pb[2];
+                        sh = E::mfma(qa[kk], kvf[kk], sh, 0, 0, 0);
+                    X8 pb[2];
     #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
     #pragma unroll
-                        for (int t = 0; t < 8; ++t) pb[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t]);
+                        for (int t = 0; t < 8; ++t) pb[ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
                     {
-                        typedef bf16x8 __attribute__((address_space(3)))* lds_b8;
+                        typedef X8 __attribute__((address_space(3)))* lds_b8;
                         const uint32_t a = px_addr + (uint32_t)((step & 1) * 64 * 32);
                         *(lds_b8)(uintptr_t)a = pb[0];
                         *(lds_b8)(uintptr_t)(a + 16) = pb[1];
                     }
                     const uint32_t dt_addr = u_addr + (uint32_t)C::TILE * 2u + col_lane;
-                    bf16x8 da[C::DT][2];
+                    X8 da[C::DT][2];
     #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
-                        for (int ks = 0; ks < 2; ++ks) da[dt][ks] = lds_column_operand_at<C::TS>(dt_addr + dt * 64, ks);
+                        for (int ks = 0; ks < 2; ++ks) da[dt][ks] = lds_column_operand_at<C::TS, X8>(dt_addr + dt * 64, ks);
     #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
                         for (int ks = 0; ks < 2; ++ks)
-                            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[dt][ks], pb[ks], oacc[dt], 0, 0, 0);
+                            oacc[dt] = E::mfma(da[dt][ks], pb[ks], oacc[dt], 0, 0, 0);
                 }
             } else {
                 // first the previous unit (its dP is still in dp_prev), then this unit's dP
                 if (act_prev) consume(slot == 0 ? C::NUNIT - 1 : slot - 1, step - 1);
                 if (act) {
                     const uint32_t d_addr = u_addr + (uint32_t)C::TILE * 2u;
-                    bf16x8 da[C::DK];
+                    X8 da[C::DK];
     #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) da[kk] = lds_read_bf16x8(d_addr + row_lane + kk * 32);
-                    dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[0], kvf[0], negr, 0, 0, 0);
+                    for (int kk = 0; kk < C::DK; ++kk) da[kk] = lds_read_x8<X8>(d_addr + row_lane + kk * 32);
+                    dp_prev = E::mfma(da[0], kvf[0], negr, 0, 0, 0);
     #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)
-                        dp_prev = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[kk], kvf[kk], dp_prev, 0, 0, 0);
+                        dp_prev = E::mfma(da[kk], kvf[kk], dp_prev, 0, 0, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
                 }
@@ -346,16 +348,16 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
-                    union { __bf16 hh[4]; uint2 u; } a;
+                    union { EL hh[4]; uint2 u; } a;
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) a.hh[x] = (__bf16)(oacc[dt][4 * g4 + x] * sc);
+                    for (int x = 0; x < 4; ++x) a.hh[x] = (EL)(oacc[dt][4 * g4 + x] * sc);
                     *(uint2*)(dst + dt * 32 + 8 * g4) = a.u;
                 }
         }
     }
 }
 
-template <int D>
+template <class E, int D>
 int launch_kv(const Problem& p, hipStream_t st) {
     using C = KvCfg<D>;
     const int njb = (p.N + VJ - 1) / VJ;
@@ -363,11 +365,11 @@ int launch_kv(const Problem& p, hipStream_t st) {
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
     const size_t lds = C::lds_bytes(p.w2);
     const bool bias = p.k2_bias != 0.f || p.v2_bias != 0.f;
-    const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<D, true> : (const void*)mfma_bwd_kv_kernel<D, false>;
+    const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<E, D, true> : (const void*)mfma_bwd_kv_kernel<E, D, false>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
-    if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<D, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
-    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<D, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
+    if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
+    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
 
@@ -375,8 +377,9 @@ int launch_kv(const Problem& p, hipStream_t st) {
 
 bool kv_fits(int D, int w2) { return D == 128 ? KvCfg<128>::fits(w2) : (D == 64 ? KvCfg<64>::fits(w2) : false); }
 
-int launch_mfma_bwd_kv(const Problem& p, hipStream_t st) {
-    return p.D == 128 ? launch_kv<128>(p, st) : launch_kv<64>(p, st);
+int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st) {
+    if (dtype == SA2_F16) return p.D == 128 ? launch_kv<ElemF16, 128>(p, st) : launch_kv<ElemF16, 64>(p, st);
+    return p.D == 128 ? launch_kv<ElemBF16, 128>(p, st) : launch_kv<ElemBF16, 64>(p, st);
 }
 
 }  // namespace sa2

@@ -1,4 +1,4 @@
-// Types and device helpers shared by the gfx950 bf16 MFMA kernels.
+// Types and device helpers shared by the gfx950 MFMA kernels (bf16 and fp16 elements).
 #pragma once
 
 #include "sa2_common.h"
@@ -9,6 +9,8 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 
 constexpr int BQ = 32;       // queries per workgroup
 constexpr int TJ = 32;       // keys per LDS tile
@@ -22,6 +24,49 @@ constexpr float LN_EPS = -18.420680743952367f;     // ln(1e-8)
 __device__ __forceinline__ float bf16_lo(uint32_t x) { return __uint_as_float(x << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// The 16-bit element type of a call: how its pairs unpack to fp32, its MFMA and its
+// two-element dot product.  WEIGHT_LIMIT bounds the row sum of one tile of softmax weights
+// in the forward's fast kernel: above it the block is recomputed by the repair kernel (bf16
+// shares fp32's exponent range; an fp16 weight must stay below 65504).
+struct ElemBF16 {
+    typedef __bf16 scalar;
+    typedef bf16x8 x8;
+    typedef bf16x2 x2;
+    static constexpr int DTYPE = SA2_BF16;
+    static constexpr float WEIGHT_LIMIT = 1.0e30f;
+    static __device__ __forceinline__ float lo(uint32_t x) { return __uint_as_float(x << 16); }
+    static __device__ __forceinline__ float hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }
+    static __device__ __forceinline__ floatx16 mfma(x8 a, x8 b, floatx16 c, int, int, int) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float dot2(x2 a, x2 b, float c, bool) {
+        return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
+    }
+};
+struct ElemF16 {
+    typedef _Float16 scalar;
+    typedef f16x8 x8;
+    typedef f16x2 x2;
+    static constexpr int DTYPE = SA2_F16;
+    static constexpr float WEIGHT_LIMIT = 3.0e4f;
+    static __device__ __forceinline__ float lo(uint32_t x) {
+        union { uint32_t u; _Float16 h[2]; } v;
+        v.u = x;
+        return (float)v.h[0];
+    }
+    static __device__ __forceinline__ float hi(uint32_t x) {
+        union { uint32_t u; _Float16 h[2]; } v;
+        v.u = x;
+        return (float)v.h[1];
+    }
+    static __device__ __forceinline__ floatx16 mfma(x8 a, x8 b, floatx16 c, int, int, int) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float dot2(x2 a, x2 b, float c, bool) {
+        return __builtin_amdgcn_fdot2(a, b, c, false);
+    }
+};
 
 // Exchange between lane l and lane l^32 (one VALU op): returns the partner's value.
 __device__ __forceinline__ float other_half(float x) {
@@ -40,13 +85,14 @@ __device__ __forceinline__ float other_half(float x) {
 // hands its values to the other operand.  Uses the LDS transpose read: within 16 lanes,
 // lane s supplies the address of row s/4, columns 4*(s%4)..+3, and lane i receives
 // column i of those four rows.
-__device__ __forceinline__ bf16x8 lds_column_operand(const uint16_t* tile, int stride, int ks, int lane) {
+template <class X8 = bf16x8>
+__device__ __forceinline__ X8 lds_column_operand(const uint16_t* tile, int stride, int ks, int lane) {
     typedef short v4s __attribute__((ext_vector_type(4)));
     const int grp = lane >> 4, s = lane & 15;
     const uint16_t* p0 = tile + (16 * ks + 4 * (grp >> 1) + (s >> 2)) * stride + 16 * (grp & 1) + 4 * (s & 3);
     const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)p0);
     const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(p0 + 8 * stride));
-    union { v4s h[2]; bf16x8 v; } u;
+    union { v4s h[2]; X8 v; } u;
     u.h[0] = a;
     u.h[1] = b;
     return u.v;
@@ -60,13 +106,13 @@ __device__ __forceinline__ uint32_t lds_column_lane_offset(int stride, int lane)
     const int grp = lane >> 4, s = lane & 15;
     return (uint32_t)(((4 * (grp >> 1) + (s >> 2)) * stride + 16 * (grp & 1) + 4 * (s & 3)) * 2);
 }
-template <int STRIDE>
-__device__ __forceinline__ bf16x8 lds_column_operand_at(uint32_t addr, int ks) {
+template <int STRIDE, class X8 = bf16x8>
+__device__ __forceinline__ X8 lds_column_operand_at(uint32_t addr, int ks) {
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef v4s __attribute__((address_space(3)))* lds_v4s;
     const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)(16 * ks * STRIDE * 2)));
     const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)((16 * ks + 8) * STRIDE * 2)));
-    union { v4s h[2]; bf16x8 v; } u;
+    union { v4s h[2]; X8 v; } u;
     u.h[0] = a;
     u.h[1] = b;
     return u.v;
@@ -115,8 +161,9 @@ __device__ __forceinline__ void lds_settle(lds_half_operand (&x)[8]) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]));
 }
-__device__ __forceinline__ bf16x8 lds_join(const lds_half_operand& a, const lds_half_operand& b) {
-    union { lds_half_operand h[2]; bf16x8 v; } u;
+template <class X8 = bf16x8>
+__device__ __forceinline__ X8 lds_join(const lds_half_operand& a, const lds_half_operand& b) {
+    union { lds_half_operand h[2]; X8 v; } u;
     u.h[0] = a;
     u.h[1] = b;
     return u.v;
@@ -125,9 +172,11 @@ __device__ __forceinline__ bf16x8 lds_join(const lds_half_operand& a, const lds_
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
-__device__ __forceinline__ bf16x8 lds_read_bf16x8(uint32_t addr) {
-    return *(const bf16x8 __attribute__((address_space(3)))*)(uintptr_t)addr;
+template <class X8 = bf16x8>
+__device__ __forceinline__ X8 lds_read_x8(uint32_t addr) {
+    return *(const X8 __attribute__((address_space(3)))*)(uintptr_t)addr;
 }
+__device__ __forceinline__ bf16x8 lds_read_bf16x8(uint32_t addr) { return lds_read_x8<bf16x8>(addr); }
 
 }  // namespace
 }  // namespace sa2

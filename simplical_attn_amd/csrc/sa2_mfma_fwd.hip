@@ -1,10 +1,10 @@
-// bf16 MFMA forward for gfx950, head_dim 64 or 128.
+// MFMA forward for gfx950 (bf16 or fp16 elements), head_dim 64 or 128.
 //
 // Formulation: expand every query i by its K' window into rows r = (i, delta),
 // delta = i - k in [0, w2], with Q~[r,:] = q[i,:] * (k2[i-delta,:] + k2_bias) *
 // scale*log2(e), rounded to bf16.  Then s[r,j] = Q~[r].k1[j] and
 // R[r,:] = sum_j p[r,j] v1[j,:] are sliding-window flash attention on the
-// expanded rows (both contractions on v_mfma_f32_32x32x16_bf16, fp32 softmax
+// expanded rows (both contractions on v_mfma_f32_32x32x16_bf16 / _f16, fp32 softmax
 // per row), and the rows of a query are merged with a second online softmax:
 // O[i] = sum_delta e^{m_r-M} (v2[i-delta]+v2_bias) * R[r] / (L + 1e-8 e^{-M}).
 // No logit outside the K' window is ever computed.
@@ -94,9 +94,12 @@ constexpr int MODE_FAST = 0, MODE_SAFE = 1, MODE_LEFT = 2;
 
 // SIDE: the K' and V' rows the block's deltas reach are copied to LDS (they fit); otherwise
 // they are read from global memory where they are needed.
-template <int D, int MODE, bool SIDE>
+template <class E, int D, int MODE, bool SIDE>
 __global__ __launch_bounds__(FT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
+    typedef typename E::scalar EL;
+    typedef typename E::x8 X8;
+    typedef typename E::x2 X2;
     constexpr bool SAFE = MODE == MODE_SAFE, LEFT = MODE == MODE_LEFT;
     static_assert(!(LEFT && SIDE), "the pre-pass keeps no row copies in LDS");
     using C = Cfg<D>;
@@ -199,12 +202,12 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             if (ACN == 8) {
                 const uint4 x = *(const uint4*)prow;
                 float* o = oacc + aq * C::OS + ac;
-                o[0] = bf16_lo(x.x); o[1] = bf16_hi(x.x); o[2] = bf16_lo(x.y); o[3] = bf16_hi(x.y);
-                o[4 % ACN] = bf16_lo(x.z); o[5 % ACN] = bf16_hi(x.z); o[6 % ACN] = bf16_lo(x.w); o[7 % ACN] = bf16_hi(x.w);
+                o[0] = E::lo(x.x); o[1] = E::hi(x.x); o[2] = E::lo(x.y); o[3] = E::hi(x.y);
+                o[4 % ACN] = E::lo(x.z); o[5 % ACN] = E::hi(x.z); o[6 % ACN] = E::lo(x.w); o[7 % ACN] = E::hi(x.w);
             } else {
                 const uint2 x = *(const uint2*)prow;
                 float* o = oacc + aq * C::OS + ac;
-                o[0] = bf16_lo(x.x); o[1] = bf16_hi(x.x); o[2] = bf16_lo(x.y); o[3] = bf16_hi(x.y);
+                o[0] = E::lo(x.x); o[1] = E::hi(x.x); o[2] = E::lo(x.y); o[3] = E::hi(x.y);
             }
             if (tid < BQ) {
                 const int it = i0 + tid < N ? i0 + tid : N - 1;
@@ -313,7 +316,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             }
         } else {
             // ---- new unit: Q~ operand, fresh softmax state ----------------------
-            bf16x8 qf[C::DK];
+            X8 qf[C::DK];
             {
                 const uint16_t* krow = k2_row(delta) + hf * 8;
                 const uint16_t* qrow;
@@ -333,11 +336,11 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                         const uint4 kb = kbv[kk];
                         const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
                         const uint32_t kw[4] = {kb.x, kb.y, kb.z, kb.w};
-                        bf16x8 r;
+                        X8 r;
 #pragma unroll
                         for (int t = 0; t < 4; ++t) {
-                            r[2 * t] = (__bf16)(bf16_lo(qw[t]) * qscale * (bf16_lo(kw[t]) + kbias));
-                            r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * qscale * (bf16_hi(kw[t]) + kbias));
+                            r[2 * t] = (EL)(E::lo(qw[t]) * qscale * (E::lo(kw[t]) + kbias));
+                            r[2 * t + 1] = (EL)(E::hi(qw[t]) * qscale * (E::hi(kw[t]) + kbias));
                         }
                         qf[kk] = r;
                     }
@@ -355,19 +358,19 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             for (int v = 0; v < 16; ++v) negm[v] = nm;
 
             // exp2 of the shifted logits -> bf16 weights (MFMA B operand) and their row sum
-            auto weights = [&](const floatx16& sh, bf16x8* w, float& rsum) {
+            auto weights = [&](const floatx16& sh, X8* w, float& rsum) {
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) w[ks][t] = (__bf16)fast_exp2(sh[ks * 8 + t]);
-                const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
+                    for (int t = 0; t < 8; ++t) w[ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
+                const X2 ones = {(EL)1.f, (EL)1.f};
                 float r = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
-                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 0, 1), ones, r, false);
-                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 2, 3), ones, r, false);
-                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 4, 5), ones, r, false);
-                    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(w[ks], w[ks], 6, 7), ones, r, false);
+                    r = E::dot2(__builtin_shufflevector(w[ks], w[ks], 0, 1), ones, r, false);
+                    r = E::dot2(__builtin_shufflevector(w[ks], w[ks], 2, 3), ones, r, false);
+                    r = E::dot2(__builtin_shufflevector(w[ks], w[ks], 4, 5), ones, r, false);
+                    r = E::dot2(__builtin_shufflevector(w[ks], w[ks], 6, 7), ones, r, false);
                 }
                 rsum = r;
             };
@@ -376,8 +379,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             auto logit_mfmas = [&](uint32_t ks_addr, floatx16 c) -> floatx16 {
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
-                    const bf16x8 ka = lds_read_bf16x8(ks_addr + k_lane + kk * KKB);
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], c, 0, 0, 0);
+                    const X8 ka = lds_read_x8<X8>(ks_addr + k_lane + kk * KKB);
+                    c = E::mfma(ka, qf[kk], c, 0, 0, 0);
                 }
                 return c;
             };
@@ -394,7 +397,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     lds_tr_issue<3 * DTB + (16 / C::RPW) * C::GROUP, 3 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[14], vh[15]);
                 }
             };
-            auto value_mfmas = [&](uint32_t vt_addr, const bf16x8* w) {
+            auto value_mfmas = [&](uint32_t vt_addr, const X8* w) {
                 lds_half_operand vh[4 * C::DT];
                 issue_v(vt_addr, vh);
                 lds_settle(vh);
@@ -402,8 +405,8 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
-                        const bf16x8 va = lds_join(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
-                        racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, w[ks], racc[dt], 0, 0, 0);
+                        const X8 va = lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
+                        racc[dt] = E::mfma(va, w[ks], racc[dt], 0, 0, 0);
                     }
             };
 
@@ -457,7 +460,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                         for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) t[v] -= m_use;
-                    bf16x8 pb[2];
+                    X8 pb[2];
                     float rs;
                     weights(t, pb, rs);
                     l += rs;
@@ -507,34 +510,34 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 auto step = [&](int s, const floatx16& prev, floatx16& cur) {
                     begin_step(s);
                     const uint32_t ks_addr = stage_addr(buf);
-                    bf16x8 ka[C::DK];
+                    X8 ka[C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_bf16x8(ks_addr + k_lane + kk * KKB);
+                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_x8<X8>(ks_addr + k_lane + kk * KKB);
                     // the reference point (and, on the two window-edge tiles, the mask) is the
                     // C operand of the first logit MFMA
                     if (__builtin_expect(tile_plain(s), 1)) {
-                        cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], negm, 0, 0, 0);
+                        cur = E::mfma(ka[0], qf[0], negm, 0, 0, 0);
                     } else {
                         asm volatile("" ::: "memory");      // keep the mask arithmetic out of the common path
-                        cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
+                        cur = E::mfma(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
                     }
                     lds_half_operand vh[4 * C::DT];
                     issue_v(vt_prev, vh);
-                    bf16x8 pb[2];
+                    X8 pb[2];
                     float rs;
 #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)
-                        cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], cur, 0, 0, 0);
+                        cur = E::mfma(ka[kk], qf[kk], cur, 0, 0, 0);
                     weights(prev, pb, rs);
                     l += rs;
-                    bad |= !(rs < OVERFLOW_LIMIT);
+                    bad |= !(rs < E::WEIGHT_LIMIT);
                     lds_settle(vh);
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) {
-                            const bf16x8 va = lds_join(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
-                            racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[ks], racc[dt], 0, 0, 0);
+                            const X8 va = lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
+                            racc[dt] = E::mfma(va, pb[ks], racc[dt], 0, 0, 0);
                         }
 #pragma unroll
                     for (int x = 1; x < C::DK; ++x) {
@@ -549,7 +552,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     step(s, sh_a, sh_b);
                     step(s + 1, sh_b, sh_a);
                 }
-                bf16x8 pb[2];
+                X8 pb[2];
                 float rs;
                 if (s <= ws1) {
                     step(s, sh_a, sh_b);
@@ -558,7 +561,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     weights(sh_a, pb, rs);
                 }
                 l += rs;
-                bad |= !(rs < OVERFLOW_LIMIT);
+                bad |= !(rs < E::WEIGHT_LIMIT);
                 value_mfmas(vt_prev - v_lane + v_lane, pb);
                 for (int s2 = ws1 + 1; s2 < nt; ++s2) {   // (pre-pass) tiles after this wavefront's window
                     begin_step(s2);
@@ -584,11 +587,11 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
                         const uint2 x = vx[4 * dt + g4];
-                        union { __bf16 h[4]; uint2 u; } o;
-                        o.h[0] = (__bf16)(inv * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + p.v2_bias));
-                        o.h[1] = (__bf16)(inv * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + p.v2_bias));
-                        o.h[2] = (__bf16)(inv * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + p.v2_bias));
-                        o.h[3] = (__bf16)(inv * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + p.v2_bias));
+                        union { EL h[4]; uint2 u; } o;
+                        o.h[0] = (EL)(inv * racc[dt][4 * g4 + 0] * (E::lo(x.x) + p.v2_bias));
+                        o.h[1] = (EL)(inv * racc[dt][4 * g4 + 1] * (E::hi(x.x) + p.v2_bias));
+                        o.h[2] = (EL)(inv * racc[dt][4 * g4 + 2] * (E::lo(x.y) + p.v2_bias));
+                        o.h[3] = (EL)(inv * racc[dt][4 * g4 + 3] * (E::hi(x.y) + p.v2_bias));
                         *(uint2*)(orow + dt * 32 + 8 * g4) = o.u;
                     }
                 if (hf == 0) {
@@ -635,7 +638,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             Lrun = Mrun > -INFINITY ? 1.f : 0.f;
         }
         const float a = fast_exp2(Mrun - Muse);
-        bad |= !(a < OVERFLOW_LIMIT);
+        bad |= !(a < E::WEIGHT_LIMIT);
         float Ln = Lrun * a;
 #pragma unroll
         for (int w = 0; w < FW; ++w) Ln += xch_l[w * BQ + ln_m] * fast_exp2(xch_m[w * BQ + ln_m] - Muse);
@@ -664,15 +667,15 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                         const uint2 x = vx[4 * dt + g4];
                         float4 o = *(float4*)(arow + dt * 32 + 8 * g4);
                         if (PLAIN) {
-                            o.x += racc[dt][4 * g4 + 0] * bf16_lo(x.x);
-                            o.y += racc[dt][4 * g4 + 1] * bf16_hi(x.x);
-                            o.z += racc[dt][4 * g4 + 2] * bf16_lo(x.y);
-                            o.w += racc[dt][4 * g4 + 3] * bf16_hi(x.y);
+                            o.x += racc[dt][4 * g4 + 0] * E::lo(x.x);
+                            o.y += racc[dt][4 * g4 + 1] * E::hi(x.x);
+                            o.z += racc[dt][4 * g4 + 2] * E::lo(x.y);
+                            o.w += racc[dt][4 * g4 + 3] * E::hi(x.y);
                         } else {
-                            o.x = o.x * a + cw * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + vb);
-                            o.y = o.y * a + cw * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + vb);
-                            o.z = o.z * a + cw * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + vb);
-                            o.w = o.w * a + cw * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + vb);
+                            o.x = o.x * a + cw * racc[dt][4 * g4 + 0] * (E::lo(x.x) + vb);
+                            o.y = o.y * a + cw * racc[dt][4 * g4 + 1] * (E::hi(x.x) + vb);
+                            o.z = o.z * a + cw * racc[dt][4 * g4 + 2] * (E::lo(x.y) + vb);
+                            o.w = o.w * a + cw * racc[dt][4 * g4 + 3] * (E::hi(x.y) + vb);
                         }
                         *(float4*)(arow + dt * 32 + 8 * g4) = o;
                     }
@@ -684,17 +687,17 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
                         const uint2 x = vx[4 * dt + g4];
-                        union { __bf16 h[4]; uint2 u; } o;
+                        union { __bf16 h[4]; uint2 u; } o;      // slabs are bf16 whatever the element type
                         if (PLAIN) {
-                            o.h[0] = (__bf16)(racc[dt][4 * g4 + 0] * bf16_lo(x.x));
-                            o.h[1] = (__bf16)(racc[dt][4 * g4 + 1] * bf16_hi(x.x));
-                            o.h[2] = (__bf16)(racc[dt][4 * g4 + 2] * bf16_lo(x.y));
-                            o.h[3] = (__bf16)(racc[dt][4 * g4 + 3] * bf16_hi(x.y));
+                            o.h[0] = (__bf16)(racc[dt][4 * g4 + 0] * E::lo(x.x));
+                            o.h[1] = (__bf16)(racc[dt][4 * g4 + 1] * E::hi(x.x));
+                            o.h[2] = (__bf16)(racc[dt][4 * g4 + 2] * E::lo(x.y));
+                            o.h[3] = (__bf16)(racc[dt][4 * g4 + 3] * E::hi(x.y));
                         } else {
-                            o.h[0] = (__bf16)(c1 * racc[dt][4 * g4 + 0] * (bf16_lo(x.x) + vb));
-                            o.h[1] = (__bf16)(c1 * racc[dt][4 * g4 + 1] * (bf16_hi(x.x) + vb));
-                            o.h[2] = (__bf16)(c1 * racc[dt][4 * g4 + 2] * (bf16_lo(x.y) + vb));
-                            o.h[3] = (__bf16)(c1 * racc[dt][4 * g4 + 3] * (bf16_hi(x.y) + vb));
+                            o.h[0] = (__bf16)(c1 * racc[dt][4 * g4 + 0] * (E::lo(x.x) + vb));
+                            o.h[1] = (__bf16)(c1 * racc[dt][4 * g4 + 1] * (E::hi(x.x) + vb));
+                            o.h[2] = (__bf16)(c1 * racc[dt][4 * g4 + 2] * (E::lo(x.y) + vb));
+                            o.h[3] = (__bf16)(c1 * racc[dt][4 * g4 + 3] * (E::hi(x.y) + vb));
                         }
                         *(uint2*)(srow + dt * 32 + 8 * g4) = o.u;
                     }
@@ -741,9 +744,9 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
         const float Ms = fin_m[aq], L = fin_l[aq];
         const float inv = 1.f / (L + 1e-8f * fast_exp2(-Ms));
         uint16_t* orow = (uint16_t*)p.out.p + p.out.off(b, io, h) + ac;
-        union { __bf16 h[8]; uint4 u4; uint2 u2; } o;
+        union { EL h[8]; uint4 u4; uint2 u2; } o;
 #pragma unroll
-        for (int c = 0; c < ACN; ++c) o.h[c] = (__bf16)(oacc[aq * C::OS + ac + c] * inv);
+        for (int c = 0; c < ACN; ++c) o.h[c] = (EL)(oacc[aq * C::OS + ac + c] * inv);
         if (ACN == 8) *(uint4*)orow = o.u4;
         else *(uint2*)orow = o.u2;
         if ((tid_f & 15) == 0) {
@@ -755,36 +758,36 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
     }
 }
 
-template <int D, bool SIDE>
+template <class E, int D, bool SIDE>
 int launch_fwd_kernels(const Problem& p, int nqb, int total, hipStream_t st) {
     using C = Cfg<D>;
     const size_t lds = C::lds_bytes(p.w2);
     // one unit left over after the rounds of eight: the pre-pass takes it
     const int left = (p.w2 >= FW && p.w2 % FW == 0) ? 1 : 0;
-    if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, MODE_FAST, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_FAST, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess ||
-        hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, MODE_SAFE, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_SAFE, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess ||
-        hipFuncSetAttribute((const void*)mfma_fwd_kernel<D, MODE_LEFT, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_LEFT, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)C::STAGE_BYTES) != hipSuccess)
         return SA2_ERR_LAUNCH_FAILED;
     if (left) {
         const int ngrp = (nqb + FW - 1) / FW;
         const int total_left = ngrp * (total / nqb);
-        hipLaunchKernelGGL((mfma_fwd_kernel<D, MODE_LEFT, false>), dim3((unsigned)total_left), dim3(FT), C::STAGE_BYTES, st, p,
+        hipLaunchKernelGGL((mfma_fwd_kernel<E, D, MODE_LEFT, false>), dim3((unsigned)total_left), dim3(FT), C::STAGE_BYTES, st, p,
                            ngrp, total_left, 0);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
-    hipLaunchKernelGGL((mfma_fwd_kernel<D, MODE_FAST, SIDE>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, left);
+    hipLaunchKernelGGL((mfma_fwd_kernel<E, D, MODE_FAST, SIDE>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, left);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL((mfma_fwd_kernel<D, MODE_SAFE, SIDE>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, left);
+    hipLaunchKernelGGL((mfma_fwd_kernel<E, D, MODE_SAFE, SIDE>), dim3((unsigned)total), dim3(FT), lds, st, p, nqb, total, left);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
 
-template <int D>
+template <class E, int D>
 int launch_fwd_pair(const Problem& p, int nqb, int total, hipStream_t st) {
-    return Cfg<D>::side_fits(p.w2) ? launch_fwd_kernels<D, true>(p, nqb, total, st)
-                                   : launch_fwd_kernels<D, false>(p, nqb, total, st);
+    return Cfg<D>::side_fits(p.w2) ? launch_fwd_kernels<E, D, true>(p, nqb, total, st)
+                                   : launch_fwd_kernels<E, D, false>(p, nqb, total, st);
 }
 
 bool aligned16(const Tensor& t, int B, int N, int H) {
@@ -802,7 +805,7 @@ bool aligned16(const Tensor& t, int B, int N, int H) {
 
 bool mfma_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
     (void)B; (void)H; (void)w1; (void)w2; (void)N;
-    return dtype == SA2_BF16 && (D == 64 || D == 128);
+    return (dtype == SA2_BF16 || dtype == SA2_F16) && (D == 64 || D == 128);
 }
 
 bool mfma_layout_ok(const Problem& p, bool backward) {
@@ -817,11 +820,13 @@ bool mfma_layout_ok(const Problem& p, bool backward) {
     return true;
 }
 
-int launch_mfma_fwd(const Problem& p, hipStream_t st) {
+int launch_mfma_fwd(const Problem& p, int dtype, hipStream_t st) {
     const int nqb = (p.N + BQ - 1) / BQ;
     const int64_t total = (int64_t)nqb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-    return p.D == 128 ? launch_fwd_pair<128>(p, nqb, (int)total, st) : launch_fwd_pair<64>(p, nqb, (int)total, st);
+    if (dtype == SA2_F16)
+        return p.D == 128 ? launch_fwd_pair<ElemF16, 128>(p, nqb, (int)total, st) : launch_fwd_pair<ElemF16, 64>(p, nqb, (int)total, st);
+    return p.D == 128 ? launch_fwd_pair<ElemBF16, 128>(p, nqb, (int)total, st) : launch_fwd_pair<ElemBF16, 64>(p, nqb, (int)total, st);
 }
 
 }  // namespace sa2

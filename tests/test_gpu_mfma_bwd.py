@@ -46,6 +46,19 @@ def test_small_shapes_vs_oracle(case):
                          atol=floor if name in ("dq", "dk1", "dk2") else 1e-6)
 
 
+@pytest.mark.parametrize("case", [SMALL[1], SMALL[6], (1, 300, 2, 64, 96, 16, 0.1, 0.0), (2, 160, 2, 128, 64, 33, 0.0, 0.0)])
+def test_small_shapes_fp16_vs_oracle(case):
+    """fp16 elements on the same kernels (fp16 MFMA).  Tolerance: max|diff| <= 1e-2 * max|ref| per
+    tensor (P, dS and the row-dot D are rounded to fp16 inside the kernels)."""
+    B, N, H, D, w1, w2, kb, vb = case
+    inp = make_inputs(B, N, H, D, seed=N + D + w1, dtype=torch.float16)
+    got = run_device(inp, w1, w2, None, kb, vb, flags=MFMA)
+    want = oracle_all(inp, w1, w2, None, kb, vb)
+    for name in GRADS:
+        assert got[name].dtype == torch.float16
+        assert_close_rel(got[name], want[name], 1e-2, name)
+
+
 def check_rows(got, inp, w1, w2, rows):
     """Oracle gradients of the loss restricted to query rows [r0, r1): complete for dq on those
     rows, and for K (K') rows whose whole forward reach [j, j+w] lies inside the range or is cut

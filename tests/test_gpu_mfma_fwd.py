@@ -1,4 +1,4 @@
-"""GPU parity of the bf16 MFMA forward kernel, through the C ABI.
+"""GPU parity of the MFMA forward kernel (bf16 and fp16 elements), through the C ABI.
 
 Tolerance (bf16 path): max|diff| <= 2e-2 * max|ref| per tensor against the
 fp64 oracle evaluated on the same bf16-rounded inputs.  Large shapes are
@@ -52,11 +52,46 @@ def test_small_shapes_vs_oracle(case):
     assert_close_rel(lse, want_lse, BF16_TOL, "lse")
 
 
+FP16_CASES = [SMALL[1], SMALL[4], SMALL[6], SMALL[7]]
+
+
+@pytest.mark.parametrize("case", FP16_CASES)
+def test_small_shapes_fp16_vs_oracle(case):
+    """fp16 elements on the same kernels (fp16 MFMA); the tolerance of the bf16 path is kept."""
+    B, N, H, D, w1, w2, kb, vb = case
+    inp = make_inputs(B, N, H, D, seed=N + D + w1, dtype=torch.float16, with_dout=False)
+    out, lse = fwd(inp, w1, w2, None, kb, vb)
+    assert out.dtype == torch.float16
+    want, want_lse = oracle_rows(inp, w1, w2, None, None, kb, vb)
+    assert_close_rel(out, want, 4e-3, "out")
+    assert_close_rel(lse, want_lse, 4e-3, "lse")
+
+
+def test_fp16_weights_beyond_half_range_go_to_the_repair_kernel():
+    """Logits that grow along the window push softmax weights (relative to the reference point
+    fixed at the first tile) past 65504: the block is recomputed with running maxima."""
+    B, N, H, D = 1, 192, 1, 64
+    g = torch.Generator().manual_seed(11)
+    q = torch.ones(B, N, H, D)
+    k2 = torch.ones(B, N, H, D)
+    ramp = torch.linspace(-1.0, 1.0, N).view(1, N, 1, 1)
+    k1 = (ramp * 4.0).expand(B, N, H, D).contiguous()           # s_ij grows with j: 64 * 4 * ramp / 8
+    v1 = torch.randn(B, N, H, D, generator=g)
+    v2 = torch.randn(B, N, H, D, generator=g)
+    inp = [t.to(torch.float16) for t in (q, k1, k2, v1, v2)]
+    out, lse = fwd(inp, 160, 8)
+    want, want_lse = oracle_rows(inp, 160, 8, None)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert_close_rel(out, want, 4e-3, "out")
+    assert_close_rel(lse, want_lse, 4e-3, "lse")
+
+
 def test_auto_dispatch_takes_mfma_for_bf16_d64_d128():
     from simplical_attn_amd import _lib
     lib = _lib.load()
     assert lib.sa2_uses_mfma(2, 2048, 8, 64, 512, 32, _lib.SA2_BF16) == 1
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_BF16) == 1
+    assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F16) == 1
     assert lib.sa2_uses_mfma(1, 128, 2, 64, 32, 16, _lib.SA2_F32) == 0
     assert lib.sa2_uses_mfma(1, 128, 2, 32, 32, 16, _lib.SA2_BF16) == 0
     inp = make_inputs(1, 96, 2, 64, seed=1, dtype=torch.bfloat16, with_dout=False)
