@@ -15,7 +15,7 @@ GENERIC = 1
 
 
 def test_config1_fp32_forward_matches_literal_oracle():
-    """BASELINE config 1: fp32, B1 H2 N128 D64, w 32/16, seed 0, rtol = atol = 1e-5
+    """Benchmark configuration 1: fp32, B1 H2 N128 D64, w 32/16, seed 0, rtol = atol = 1e-5
     against the literal-order fp32 loop and against the fp64 truth."""
     inp = make_inputs(1, 128, 2, 64, seed=0)
     got = run_device(inp, 32, 16, flags=GENERIC, backward=False)

@@ -86,17 +86,17 @@ def check_large(B, N, H, D, w1, w2, seed, rows, qk_mag=None, more_rows=(), gener
 
 
 def test_config3_forward_backward():
-    """BASELINE config 3: bf16, B2 H8 N2048 D64, w 512/32, seed 2."""
+    """Benchmark configuration 3: bf16, B2 H8 N2048 D64, w 512/32, seed 2."""
     check_large(2, 2048, 8, 64, 512, 32, seed=2, rows=(0, 640))
 
 
 def test_config4_headline_shape_gradients():
-    """BASELINE config 4: bf16, B1 H16 N8192 D128, w 512/32, seed 3."""
+    """Benchmark configuration 4: bf16, B1 H16 N8192 D128, w 512/32, seed 3."""
     check_large(1, 8192, 16, 128, 512, 32, seed=3, rows=(448, 1088))
 
 
 def test_config5_long_sequence_gradients():
-    """BASELINE config 5: bf16, B1 H8 N32768 D128, w 1024/64, q/k/k' ~ N(0, 0.5^2), seed 4.  Checked
+    """Benchmark configuration 5: bf16, B1 H8 N32768 D128, w 1024/64, q/k/k' ~ N(0, 0.5^2), seed 4.  Checked
     on query rows around i = w1 and at the end of the sequence (the generic kernels would take
     minutes at this size)."""
     check_large(1, 32768, 8, 128, 1024, 64, seed=4, rows=(992, 2048), qk_mag=0.5,

@@ -101,7 +101,7 @@ def test_auto_dispatch_takes_mfma_for_bf16_d64_d128():
 
 
 def test_config2_forward():
-    """BASELINE config 2: bf16, B2 H8 N2048 D64, w 512/32, seed 1."""
+    """Benchmark configuration 2: bf16, B2 H8 N2048 D64, w 512/32, seed 1."""
     inp = make_inputs(2, 2048, 8, 64, seed=1, dtype=torch.bfloat16, with_dout=False)
     out, lse = fwd(inp, 512, 32)
     for rows in ((0, 96), (480, 576), (1990, 2048)):
@@ -114,7 +114,7 @@ def test_config2_forward():
 
 
 def test_config4_forward_headline_shape():
-    """BASELINE config 4: bf16, B1 H16 N8192 D128, w 512/32, seed 3; oracle on
+    """Benchmark configuration 4: bf16, B1 H16 N8192 D128, w 512/32, seed 3; oracle on
     row ranges (start, the block straddling i = w1, end), generic kernel on all rows."""
     inp = make_inputs(1, 8192, 16, 128, seed=3, dtype=torch.bfloat16, with_dout=False)
     out, lse = fwd(inp, 512, 32)
