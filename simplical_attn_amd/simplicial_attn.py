@@ -145,6 +145,55 @@ class TwoSimplicialAttentionFunction(torch.autograd.Function):
         return (*grads, None, None, None, None, None)
 
 
+class _ExactFunction(torch.autograd.Function):
+    """The same operator on the fp32 FMA kernels (every product and sum in fp32, whatever the
+    element type of the tensors): the slow, exact path that plays the part of the reference's
+    PyTorch loop when results of the MFMA kernels are to be checked on the device."""
+
+    @staticmethod
+    def forward(ctx, q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias):
+        if scale is None:
+            scale = 1.0 / math.sqrt(q.shape[-1])
+        out, lse = simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias, _lib.FLAG_FORCE_GENERIC)
+        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse)
+        ctx.w1, ctx.w2, ctx.scale, ctx.k2_bias, ctx.v2_bias = w1, w2, scale, k2_bias, v2_bias
+        ctx.window_inclusive = WINDOW_INCLUSIVE
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k1, k2, v1, v2, out, lse = ctx.saved_tensors
+        grads = simplicial_backward(q, k1, k2, v1, v2, out, lse, grad_output, ctx.w1, ctx.w2, ctx.scale,
+                                    ctx.k2_bias, ctx.v2_bias, needs=tuple(ctx.needs_input_grad[:5]),
+                                    flags=_lib.FLAG_FORCE_GENERIC, window_inclusive=ctx.window_inclusive)
+        return (*grads, None, None, None, None, None)
+
+
+def two_simplicial_attention_reference(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0):
+    """Signature of the reference's PyTorch implementation (simplicial/reference.py:8-9).  Here it
+    runs the fp32 FMA kernels on the GPU (same windows, bias and epsilon as reference.py:27-76) and
+    is differentiable; it is the device-side yardstick for the MFMA kernels, not a CPU path."""
+    return _ExactFunction.apply(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias)
+
+
+class TwoSimplicialAttentionReference(torch.nn.Module):
+    """Module wrapper of two_simplicial_attention_reference with the reference's constructor
+    (simplicial/reference.py:79-103)."""
+
+    def __init__(self, head_dim, w1=64, w2=64, scale=None, k2_bias=0.0, v2_bias=0.0):
+        super().__init__()
+        self.head_dim = head_dim
+        self.w1 = w1
+        self.w2 = w2
+        self.scale = scale if scale is not None else (1.0 / math.sqrt(head_dim))
+        self.k2_bias = k2_bias
+        self.v2_bias = v2_bias
+
+    def forward(self, q, k1, k2, v1, v2):
+        return two_simplicial_attention_reference(q, k1, k2, v1, v2, self.w1, self.w2, self.scale,
+                                                  self.k2_bias, self.v2_bias)
+
+
 class TwoSimplicialAttention(torch.nn.Module):
     """Module wrapper with the reference's constructor and call signature
     (simplicial/triton_impl.py:161-186); holds no parameters."""

@@ -191,6 +191,24 @@ def test_error_codes():
         simplicial_forward(y.cpu(), y.cpu(), y.cpu(), y.cpu(), y.cpu(), 4, 4)
 
 
+def test_reference_named_entry_points_run_the_exact_kernels():
+    """two_simplicial_attention_reference / TwoSimplicialAttentionReference (the reference's names,
+    simplicial/reference.py:8, 79): bf16 tensors, fp32 arithmetic, differentiable; they agree with
+    the oracle more closely than the bf16 parity bar and with the MFMA kernels within it."""
+    import simplical_attn_amd as sa
+    dev = torch.device("cuda:0")
+    inp = make_inputs(1, 96, 2, 64, seed=9, dtype=torch.bfloat16)
+    leaves = [x.to(dev).requires_grad_(True) for x in inp[:5]]
+    out = sa.TwoSimplicialAttentionReference(64, 20, 6, k2_bias=0.1)(*leaves)
+    out.backward(inp[5].to(dev))
+    want = oracle_all(inp, 20, 6, None, 0.1, 0.0)
+    assert_close_rel(out, want["out"], 5e-3, "out")
+    for name, leaf in zip(("dq", "dk1", "dk2", "dv1", "dv2"), leaves):
+        assert_close_rel(leaf.grad, want[name], 1e-2, name)
+    fast = sa.TwoSimplicialAttention(64, 20, 6, k2_bias=0.1)(*[x.to(dev) for x in inp[:5]])
+    assert_close_rel(fast, out.detach().float().cpu(), 2e-2, "mfma vs exact kernels")
+
+
 def test_rowdot():
     from simplical_attn_amd import compute_D_kernel
     dev = torch.device("cuda:0")
