@@ -119,3 +119,27 @@ def test_needs_input_grad_subsets_and_determinism():
                 assert torch.equal(leaves[t].grad, full[name]), name
             else:
                 assert leaves[t].grad is None
+
+
+def test_headline_shape_scaling_and_swap_properties():
+    """Size-independent checks at the headline shape (bf16 B1 H16 N8192 D128 w 512/32), whole
+    tensors.  (1) Doubling v1 is exact in bf16 and in every fp32 sum, so out, dq, dk1, dk2 and dv2
+    must double bit for bit while lse and dv1 must not change at all.  (2) With w1 = w2 the operator
+    is symmetric under (k1, v1) <-> (k2, v2): outputs agree within the bf16 bar and the gradient
+    pairs swap (the two sides run through different kernels)."""
+    inp = make_inputs(1, 8192, 16, 128, seed=3, dtype=torch.bfloat16)
+    a = run_device(inp, 512, 32, flags=MFMA)
+    inp2 = list(inp)
+    inp2[3] = inp[3] * 2
+    b = run_device(inp2, 512, 32, flags=MFMA)
+    assert torch.equal(b["lse"], a["lse"]) and torch.equal(b["dv1"], a["dv1"])
+    for name in ("out", "dq", "dk1", "dk2", "dv2"):
+        assert torch.equal(b[name], a[name] * 2), name
+    w = 64
+    small = [x[:, :2048, :4].contiguous() for x in inp]
+    c = run_device(small, w, w, flags=MFMA)
+    q, k1, k2, v1, v2, dout = small
+    d = run_device([q, k2, k1, v2, v1, dout], w, w, flags=MFMA)
+    assert_close_rel(d["out"], c["out"].float().cpu(), BF16_TOL, "out under swap")
+    for x, y in (("dq", "dq"), ("dk1", "dk2"), ("dk2", "dk1"), ("dv1", "dv2"), ("dv2", "dv1")):
+        assert_close_rel(d[x], c[y].float().cpu(), BF16_TOL, "%s under swap" % x)
