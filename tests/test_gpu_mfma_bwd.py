@@ -143,3 +143,29 @@ def test_headline_shape_scaling_and_swap_properties():
     assert_close_rel(d["out"], c["out"].float().cpu(), BF16_TOL, "out under swap")
     for x, y in (("dq", "dq"), ("dk1", "dk2"), ("dk2", "dk1"), ("dv1", "dv2"), ("dv2", "dv1")):
         assert_close_rel(d[x], c[y].float().cpu(), BF16_TOL, "%s under swap" % x)
+
+
+def test_packed_projection_views_take_the_mfma_kernels():
+    """q, k1, k2, v1, v2 as slices of one [B, N, 5, H, D] projection output (row stride 5*H*D, no
+    copies): the MFMA kernels take per-tensor strides, and every result equals the one from
+    contiguous copies bit for bit."""
+    import simplical_attn_amd as sa
+    from simplical_attn_amd import _lib
+    dev = torch.device("cuda:0")
+    B, N, H, D, w1, w2 = 2, 200, 3, 128, 70, 12
+    g = torch.Generator().manual_seed(77)
+    packed = torch.randn(B, N, 5, H, D, generator=g).to(torch.bfloat16).to(dev)
+    dout = torch.randn(B, N, H, D, generator=g).to(torch.bfloat16).to(dev)
+    views = [packed[:, :, t] for t in range(5)]
+    assert all(not v.is_contiguous() for v in views)
+    out_v, lse_v = sa.simplicial_forward(*views, w1, w2, flags=_lib.FLAG_FORCE_MFMA)
+    grads_v = sa.simplicial_backward(*views, out_v, lse_v, dout, w1, w2, flags=_lib.FLAG_FORCE_MFMA)
+    copies = [v.contiguous() for v in views]
+    out_c, lse_c = sa.simplicial_forward(*copies, w1, w2, flags=_lib.FLAG_FORCE_MFMA)
+    grads_c = sa.simplicial_backward(*copies, out_c, lse_c, dout, w1, w2, flags=_lib.FLAG_FORCE_MFMA)
+    assert torch.equal(out_v, out_c) and torch.equal(lse_v, lse_c)
+    for a, b in zip(grads_v, grads_c):
+        assert torch.equal(a, b)
+    want = oracle_all([c.cpu() for c in copies] + [dout.cpu()], w1, w2)
+    assert_close_rel(out_v, want["out"], BF16_TOL, "out")
+    assert_close_rel(grads_v[0], want["dq"], BF16_TOL, "dq")
