@@ -44,9 +44,9 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 967.0e6,                # pre-pass 522.5 MB + fast kernel 443.4 MB + repair launch 1.1 MB
-    ("c4", "backward_k_side"): 620.9e6,        # mfma_bwd_kv_kernel
-    ("c4", "backward_kprime_side"): 1948.3e6,  # pre-pass 759.6 MB + mfma_bwd_kp_kernel 887.1 MB + dq_sum 301.6 MB
+    ("c4", "forward"): 859.0e6,                # pre-pass 413.8 MB + fast kernel 444.1 MB + repair launch 1.1 MB
+    ("c4", "backward_k_side"): 603.4e6,        # mfma_bwd_kv_kernel
+    ("c4", "backward_kprime_side"): 1953.3e6,  # pre-pass 764.8 MB + mfma_bwd_kp_kernel 887.0 MB + dq_sum 301.5 MB
 }
 
 
