@@ -47,7 +47,7 @@ typedef enum sa2_dtype { SA2_F32 = 0, SA2_BF16 = 1, SA2_F16 = 2 } sa2_dtype;
 /* flags */
 #define SA2_FLAG_AUTO 0u            /* MFMA kernels when the shape allows, generic otherwise */
 #define SA2_FLAG_FORCE_GENERIC 1u   /* fp32-FMA kernels (any dtype, any D <= 256) */
-#define SA2_FLAG_FORCE_MFMA 2u      /* bf16 MFMA kernels or SA2_ERR_UNSUPPORTED */
+#define SA2_FLAG_FORCE_MFMA 2u      /* MFMA kernels (bf16 or fp16, D 64 or 128) or SA2_ERR_UNSUPPORTED */
 
 /* Tensor order of the `strides` argument (3 int64 per tensor: batch, sequence, head). */
 enum { SA2_T_Q = 0, SA2_T_K1, SA2_T_K2, SA2_T_V1, SA2_T_V2, SA2_T_OUT, SA2_FWD_TENSORS,
@@ -60,7 +60,7 @@ int sa2_version(void);
 /* Static, NUL-terminated description of a status code. */
 const char* sa2_strerror(int status);
 
-/* 1 if sa2_forward / sa2_backward would take the bf16 MFMA kernels for this
+/* 1 if sa2_forward / sa2_backward would take the MFMA kernels for this
  * problem under SA2_FLAG_AUTO, 0 if they would take the generic kernels. */
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype);
 
@@ -73,6 +73,8 @@ int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype);
  *   lse            [B,H,N] fp32, natural-log LSE        (triton_impl.py:24)
  *   strides        SA2_FWD_TENSORS x 3 element strides  (HOST pointer)
  *   window_inclusive  1: windows [i-w, i] (reference.py); 0: (i-w, i] (kernels.py:133-136)
+ * While the call runs, `out` and `lse` also hold intermediate results of its first kernel: their
+ * contents are final only once the call's work on the stream has completed.
  */
 int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
                 void* out, float* lse,
@@ -93,7 +95,8 @@ size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int d
  *   out, dout, lse   forward output, upstream gradient, forward LSE
  *   dq,dk1,dk2,dv1,dv2  gradients in `dtype`; a NULL pointer means "not needed"
  *                       (ctx.needs_input_grad, triton_impl.py:73-77); every
- *                       non-NULL gradient is fully overwritten (no pre-zeroing needed)
+ *                       non-NULL gradient is fully overwritten (no pre-zeroing needed; dk2 and
+ *                       dv2 also hold intermediate results while the call runs)
  *   workspace        >= sa2_bwd_workspace_bytes(...) bytes, 256-byte aligned; contents
  *                    on entry are ignored
  *   strides          SA2_BWD_TENSORS x 3 element strides (HOST pointer)
