@@ -107,6 +107,8 @@ int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, c
     p.out = make_tensor(out, strides, SA2_T_OUT);
     p.lse = lse;
 
+    p.force_prepass = (flags & SA2_FLAG_FORCE_MFMA) ? 1 : 0;
+
     hipStream_t st = (hipStream_t)hip_stream;
     const bool mfma = pick_mfma(p, dtype, flags, false, &rc);
     if (rc != SA2_OK) return rc;
@@ -162,6 +164,8 @@ int sa2_backward(const void* q, const void* k1, const void* k2, const void* v1, 
     p.dsum = (float*)workspace;
     p.scratch = (char*)workspace + dsum_bytes(B, N, H);
     p.scratch_bytes = workspace_bytes - dsum_bytes(B, N, H);
+
+    p.force_prepass = (flags & SA2_FLAG_FORCE_MFMA) ? 1 : 0;
 
     hipStream_t st = (hipStream_t)hip_stream;
     const bool mfma = pick_mfma(p, dtype, flags, true, &rc);

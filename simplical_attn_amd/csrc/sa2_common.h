@@ -27,6 +27,7 @@ struct Problem {
     float* dsum;                     // [B,H,N]  sum_d dout*out
     void* scratch;                   // remaining workspace (path specific)
     size_t scratch_bytes;
+    int force_prepass;               // take the pre-pass kernels whenever the window allows, whatever the size
 };
 
 // ---- element loads / stores -------------------------------------------------

@@ -741,7 +741,8 @@ int launch_kp(const Problem& p, hipStream_t st) {
     const size_t lds = C::lds_bytes(p.w2, raw);
     float* part = (float*)p.scratch;
     // one unit left over after the rounds of four: the pre-pass takes it
-    const int left = (p.w2 >= NPAIR && p.w2 % NPAIR == 0) ? 1 : 0;
+    // (unless the grid is so small that a further launch costs more than the lone round)
+    const int left = (p.w2 >= NPAIR && p.w2 % NPAIR == 0 && (p.force_prepass || total >= 768)) ? 1 : 0;
     if (left) {
         const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + C::PX_BYTES;
         const int ngrp = (nkb + NPAIR - 1) / NPAIR;

@@ -91,6 +91,7 @@ struct Cfg {
 // R * (v2 + bias) / l in bf16 and to `lse` as m + log2(l); the fast kernel, launched next with
 // left = 1, starts its accumulator from that pair and handles delta < w2 in full rounds.
 constexpr int MODE_FAST = 0, MODE_SAFE = 1, MODE_LEFT = 2;
+constexpr int PREPASS_MIN_WORKGROUPS = 768;      // three workgroups per CU
 
 // SIDE: the K' and V' rows the block's deltas reach are copied to LDS (they fit); otherwise
 // they are read from global memory where they are needed.
@@ -762,8 +763,9 @@ template <class E, int D, bool SIDE>
 int launch_fwd_kernels(const Problem& p, int nqb, int total, hipStream_t st) {
     using C = Cfg<D>;
     const size_t lds = C::lds_bytes(p.w2);
-    // one unit left over after the rounds of eight: the pre-pass takes it
-    const int left = (p.w2 >= FW && p.w2 % FW == 0) ? 1 : 0;
+    // one unit left over after the rounds of eight: the pre-pass takes it, unless the grid is so
+    // small that a further launch costs more than the lone round
+    const int left = (p.w2 >= FW && p.w2 % FW == 0 && (p.force_prepass || total >= PREPASS_MIN_WORKGROUPS)) ? 1 : 0;
     if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_FAST, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess ||
         hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_SAFE, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
