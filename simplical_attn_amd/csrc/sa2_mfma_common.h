@@ -15,7 +15,6 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 constexpr int BQ = 32;       // queries per workgroup
 constexpr int TJ = 32;       // keys per LDS tile
 constexpr int NTHREADS = 256;
-constexpr float OVERFLOW_LIMIT = 1.0e30f;    // a row sum above this means a stale softmax reference point
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 constexpr float LOG2_EPS = -26.575424759098897f;   // log2(1e-8)
@@ -76,29 +75,15 @@ __device__ __forceinline__ float other_half(float x) {
     return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
 }
 
-// Eight bf16 of one COLUMN of a row-major [row][col] bf16 tile in LDS, as the A/B operand
-// of a 32x32x16 MFMA whose contraction index runs over the tile's rows.  `tile` points at
-// the tile's 32x32 sub-block (rows r0.., columns c0..), `stride` is the row stride in
-// elements.  Lane l gets column c0 + l%32 and, for its half h = l/32, the rows
+// Eight 16-bit elements of one COLUMN of a row-major [row][col] tile in LDS, as the A/B operand
+// of a 32x32x16 MFMA whose contraction index runs over the tile's rows, for the tile's
+// 32x32 sub-block at rows r0.., columns c0.. (`stride` = row stride in elements).  Lane l gets column c0 + l%32 and, for its half h = l/32, the rows
 //   r0 + 16*ks + 4*h + {0,1,2,3}   and   r0 + 16*ks + 8 + 4*h + {0,1,2,3}
 // which is exactly the k-slot order in which a 32x32 accumulator tile (rows = those rows)
 // hands its values to the other operand.  Uses the LDS transpose read: within 16 lanes,
 // lane s supplies the address of row s/4, columns 4*(s%4)..+3, and lane i receives
 // column i of those four rows.
-template <class X8 = bf16x8>
-__device__ __forceinline__ X8 lds_column_operand(const uint16_t* tile, int stride, int ks, int lane) {
-    typedef short v4s __attribute__((ext_vector_type(4)));
-    const int grp = lane >> 4, s = lane & 15;
-    const uint16_t* p0 = tile + (16 * ks + 4 * (grp >> 1) + (s >> 2)) * stride + 16 * (grp & 1) + 4 * (s & 3);
-    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)p0);
-    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(p0 + 8 * stride));
-    union { v4s h[2]; X8 v; } u;
-    u.h[0] = a;
-    u.h[1] = b;
-    return u.v;
-}
-
-// The same operand from LDS byte addresses.  lds_column_lane_offset() is the per-lane part
+// The operand is read from LDS byte addresses.  lds_column_lane_offset() is the per-lane part
 // (bytes, for ks = 0, relative to the 32x32 sub-block); lds_column_operand_at() takes the sum of
 // the sub-block's LDS byte address and that lane part, so that inside a loop the address is one
 // add and everything else sits in the instructions' immediate offsets.
@@ -120,7 +105,7 @@ __device__ __forceinline__ X8 lds_column_operand_at(uint32_t addr, int ks) {
 // Tiles written by direct global->LDS loads keep groups of RPW rows together: within a group
 // the 16-byte chunk c of row q sits at byte (c * RPW + q) * 16, groups lie GROUP bytes apart.
 // Transposed MFMA operand out of such a tile (same lanes and k-slot order as
-// lds_column_operand): the lane part of the address, and the two reads of k-step ks of the
+// lds_column_operand_at): the lane part of the address, and the two reads of k-step ks of the
 // 32-column block whose byte address (block * 64 * RPW) is already in `addr`.
 template <int RPW, int GROUP>
 __device__ __forceinline__ uint32_t lds_group_column_lane_offset(int lane) {
@@ -128,17 +113,6 @@ __device__ __forceinline__ uint32_t lds_group_column_lane_offset(int lane) {
     const int rr = 4 * (grp >> 1) + (s >> 2);            // row within the 8-row slice
     const int cc = 16 * (grp & 1) + 4 * (s & 3);         // column within the 32-column block
     return (uint32_t)((rr / RPW) * GROUP + ((cc / 8) * RPW + rr % RPW) * 16 + (cc % 8) * 2);
-}
-template <int RPW, int GROUP>
-__device__ __forceinline__ bf16x8 lds_group_column_operand(uint32_t addr, int ks) {
-    typedef short v4s __attribute__((ext_vector_type(4)));
-    typedef v4s __attribute__((address_space(3)))* lds_v4s;
-    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)((16 * ks / RPW) * GROUP)));
-    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)(((16 * ks + 8) / RPW) * GROUP)));
-    union { v4s h[2]; bf16x8 v; } u;
-    u.h[0] = a;
-    u.h[1] = b;
-    return u.v;
 }
 // The same operand read in two phases for loops that keep direct global->LDS loads in
 // flight: the compiler would wait for every outstanding vector-memory operation before a
@@ -176,7 +150,6 @@ template <class X8 = bf16x8>
 __device__ __forceinline__ X8 lds_read_x8(uint32_t addr) {
     return *(const X8 __attribute__((address_space(3)))*)(uintptr_t)addr;
 }
-__device__ __forceinline__ bf16x8 lds_read_bf16x8(uint32_t addr) { return lds_read_x8<bf16x8>(addr); }
 
 }  // namespace
 }  // namespace sa2
