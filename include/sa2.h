@@ -47,7 +47,7 @@ typedef enum sa2_dtype { SA2_F32 = 0, SA2_BF16 = 1, SA2_F16 = 2 } sa2_dtype;
 /* flags */
 #define SA2_FLAG_AUTO 0u            /* MFMA kernels when the shape allows, generic otherwise */
 #define SA2_FLAG_FORCE_GENERIC 1u   /* fp32-FMA kernels (any dtype, any D <= 256) */
-#define SA2_FLAG_FORCE_MFMA 2u      /* MFMA kernels (bf16 or fp16, D 64 or 128) or SA2_ERR_UNSUPPORTED; also takes
+#define SA2_FLAG_FORCE_MFMA 2u      /* MFMA kernels (bf16 or fp16, D 32, 64 or 128) or SA2_ERR_UNSUPPORTED; also takes
                                        their pre-pass kernels whenever the window sizes allow, whatever the
                                        problem size (SA2_FLAG_AUTO leaves them out for small grids) */
 

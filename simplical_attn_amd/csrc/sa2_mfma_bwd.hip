@@ -617,8 +617,8 @@ int launch_row_part(const Problem& p, hipStream_t st) {
 
 bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
     if (!mfma_supported(B, N, H, D, w1, w2, dtype)) return false;
-    // the workspace fallback kernels for wide K' windows exist for bf16 only
-    return dtype == SA2_BF16 || (kp_fits(D, w2) && kv_fits(D, w2));
+    // the workspace fallback kernels for wide K' windows exist for bf16 with D = 64 or 128 only
+    return (dtype == SA2_BF16 && D != 32) || (kp_fits(D, w2) && kv_fits(D, w2));
 }
 
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {

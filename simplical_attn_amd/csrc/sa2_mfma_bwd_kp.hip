@@ -46,6 +46,8 @@ struct KpCfg {
     // group of RPW rows (1 KB), lane L putting the 16-byte chunk L / RPW of row L % RPW at byte
     // 16 * L; groups lie GROUP bytes apart.  Row and transposed operand reads are conflict free.
     static constexpr int RPW = 512 / D;
+    // byte offset of row r of a tile (chunk 0)
+    static constexpr int row_off(int r) { return (r / RPW) * GROUP + (r % RPW) * 16; }
     static constexpr int GROUP = 1024 + 16 * RPW;
     static constexpr int NGROUP = TJ / RPW;
     static constexpr int TILE_BYTES = NGROUP * GROUP;
@@ -240,13 +242,15 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const uint32_t row_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);   // row operand
     const uint32_t col_lane = lds_group_column_lane_offset<C::RPW, C::GROUP>(lane);                      // transposed operand
     constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;      // operand strides of a k-step / a 32-column block
-    constexpr uint32_t GA = (16 / C::RPW) * C::GROUP, GB = (8 / C::RPW) * C::GROUP;
+    constexpr uint32_t GA = C::row_off(16), GB = C::row_off(8);
     // all transposed operand reads of a tile (opaque reads, settled before use)
     auto issue_tr = [&](uint32_t a, lds_half_operand (&h)[4 * C::DT]) {
         lds_tr_issue<0, GB>(a, h[0], h[1]);
         lds_tr_issue<GA, GA + GB>(a, h[2], h[3]);
-        lds_tr_issue<DTB, DTB + GB>(a, h[4], h[5]);
-        lds_tr_issue<DTB + GA, DTB + GA + GB>(a, h[6], h[7]);
+        if constexpr (C::DT >= 2) {
+            lds_tr_issue<DTB, DTB + GB>(a, h[4], h[5]);
+            lds_tr_issue<DTB + GA, DTB + GA + GB>(a, h[6], h[7]);
+        }
         if constexpr (C::DT == 4) {
             lds_tr_issue<2 * DTB, 2 * DTB + GB>(a, h[8], h[9]);
             lds_tr_issue<2 * DTB + GA, 2 * DTB + GA + GB>(a, h[10], h[11]);
@@ -602,24 +606,28 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                             constexpr int NV = C::DK / 2;             // float4 slots of this phase
                             float4 a[NV];
                             uint2 x[NV];
+                            // slot e of the phase -> 32-column tile dt and 8-column group g4 (D = 32
+                            // has one tile: the four phases take its four groups)
+                            auto slot_dt = [&](int e) { return D == 32 ? 0 : (((P0 + t) & 3) + 4 * (e >> 1)) >> 1; };
+                            auto slot_g4 = [&](int e) {
+                                return D == 32 ? ((P0 + t) & 3) : 2 * ((((P0 + t) & 3) + 4 * (e >> 1)) & 1) + (e & 1);
+                            };
 #pragma unroll
                             for (int e = 0; e < NV; ++e) {
-                                const int sb16 = ((P0 + t) & 3) + 4 * (e >> 1);
-                                const int col = (sb16 >> 1) * 32 + 8 * (2 * (sb16 & 1) + (e & 1));
+                                const int col = slot_dt(e) * 32 + 8 * slot_g4(e);
                                 x[e] = *(const uint2*)(krow + col);
                                 a[e] = *(float4*)(arow + col);
                             }
                             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                             for (int e = 0; e < NV; ++e) {
-                                const int sb16 = ((P0 + t) & 3) + 4 * (e >> 1);
-                                const int dt = sb16 >> 1, g4 = 2 * (sb16 & 1) + (e & 1);
+                                const int dt = slot_dt(e), g4 = slot_g4(e);
                                 const float kb = WITH_BIAS ? p.k2_bias : 0.f;
                                 a[e].x += gacc[dt][4 * g4 + 0] * (E::lo(x[e].x) + kb);
                                 a[e].y += gacc[dt][4 * g4 + 1] * (E::hi(x[e].x) + kb);
                                 a[e].z += gacc[dt][4 * g4 + 2] * (E::lo(x[e].y) + kb);
                                 a[e].w += gacc[dt][4 * g4 + 3] * (E::hi(x[e].y) + kb);
-                                *(float4*)(arow + (sb16 >> 1) * 32 + 8 * g4) = a[e];
+                                *(float4*)(arow + dt * 32 + 8 * g4) = a[e];
                             }
                         }
                         if (t < 3) __syncthreads();
@@ -771,7 +779,9 @@ int launch_kp(const Problem& p, hipStream_t st) {
 
 }  // namespace
 
-bool kp_fits(int D, int w2) { return D == 128 ? KpCfg<128>::fits(w2) : (D == 64 ? KpCfg<64>::fits(w2) : false); }
+bool kp_fits(int D, int w2) {
+    return D == 128 ? KpCfg<128>::fits(w2) : D == 64 ? KpCfg<64>::fits(w2) : D == 32 ? KpCfg<32>::fits(w2) : false;
+}
 
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {
     const size_t nkb = (size_t)(N + BQ - 1) / BQ;
@@ -779,8 +789,9 @@ size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {
 }
 
 int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st) {
-    if (dtype == SA2_F16) return p.D == 128 ? launch_kp<ElemF16, 128>(p, st) : launch_kp<ElemF16, 64>(p, st);
-    return p.D == 128 ? launch_kp<ElemBF16, 128>(p, st) : launch_kp<ElemBF16, 64>(p, st);
+    if (dtype == SA2_F16)
+        return p.D == 128 ? launch_kp<ElemF16, 128>(p, st) : p.D == 64 ? launch_kp<ElemF16, 64>(p, st) : launch_kp<ElemF16, 32>(p, st);
+    return p.D == 128 ? launch_kp<ElemBF16, 128>(p, st) : p.D == 64 ? launch_kp<ElemBF16, 64>(p, st) : launch_kp<ElemBF16, 32>(p, st);
 }
 
 }  // namespace sa2

@@ -375,11 +375,14 @@ int launch_kv(const Problem& p, hipStream_t st) {
 
 }  // namespace
 
-bool kv_fits(int D, int w2) { return D == 128 ? KvCfg<128>::fits(w2) : (D == 64 ? KvCfg<64>::fits(w2) : false); }
+bool kv_fits(int D, int w2) {
+    return D == 128 ? KvCfg<128>::fits(w2) : D == 64 ? KvCfg<64>::fits(w2) : D == 32 ? KvCfg<32>::fits(w2) : false;
+}
 
 int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st) {
-    if (dtype == SA2_F16) return p.D == 128 ? launch_kv<ElemF16, 128>(p, st) : launch_kv<ElemF16, 64>(p, st);
-    return p.D == 128 ? launch_kv<ElemBF16, 128>(p, st) : launch_kv<ElemBF16, 64>(p, st);
+    if (dtype == SA2_F16)
+        return p.D == 128 ? launch_kv<ElemF16, 128>(p, st) : p.D == 64 ? launch_kv<ElemF16, 64>(p, st) : launch_kv<ElemF16, 32>(p, st);
+    return p.D == 128 ? launch_kv<ElemBF16, 128>(p, st) : p.D == 64 ? launch_kv<ElemBF16, 64>(p, st) : launch_kv<ElemBF16, 32>(p, st);
 }
 
 }  // namespace sa2

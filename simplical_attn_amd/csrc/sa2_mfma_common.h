@@ -131,6 +131,9 @@ __device__ __forceinline__ void lds_settle(lds_half_operand (&x)[16]) {
                  : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]),
                    "+v"(x[8]), "+v"(x[9]), "+v"(x[10]), "+v"(x[11]), "+v"(x[12]), "+v"(x[13]), "+v"(x[14]), "+v"(x[15]));
 }
+__device__ __forceinline__ void lds_settle(lds_half_operand (&x)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]));
+}
 __device__ __forceinline__ void lds_settle(lds_half_operand (&x)[8]) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]));
@@ -141,6 +144,27 @@ __device__ __forceinline__ X8 lds_join(const lds_half_operand& a, const lds_half
     u.h[0] = a;
     u.h[1] = b;
     return u.v;
+}
+// NW consecutive 32-bit words (2*NW 16-bit elements) from / to a NW*4-byte aligned address
+template <int NW>
+__device__ __forceinline__ void load_words(const void* p, uint32_t (&w)[NW]) {
+    static_assert(NW == 1 || NW == 2 || NW == 4, "one 4-, 8- or 16-byte access");
+    if constexpr (NW == 4) {
+        const uint4 x = *(const uint4*)p;
+        w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
+    } else if constexpr (NW == 2) {
+        const uint2 x = *(const uint2*)p;
+        w[0] = x.x; w[1] = x.y;
+    } else {
+        w[0] = *(const uint32_t*)p;
+    }
+}
+template <int NW>
+__device__ __forceinline__ void store_words(void* p, const uint32_t (&w)[NW]) {
+    static_assert(NW == 1 || NW == 2 || NW == 4, "one 4-, 8- or 16-byte access");
+    if constexpr (NW == 4) *(uint4*)p = make_uint4(w[0], w[1], w[2], w[3]);
+    else if constexpr (NW == 2) *(uint2*)p = make_uint2(w[0], w[1]);
+    else *(uint32_t*)p = w[0];
 }
 // LDS byte address of a pointer into shared memory
 __device__ __forceinline__ uint32_t lds_address(const void* p) {

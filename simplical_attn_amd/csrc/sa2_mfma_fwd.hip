@@ -1,4 +1,4 @@
-// MFMA forward for gfx950 (bf16 or fp16 elements), head_dim 64 or 128.
+// MFMA forward for gfx950 (bf16 or fp16 elements), head_dim 32, 64 or 128.
 //
 // Formulation: expand every query i by its K' window into rows r = (i, delta),
 // delta = i - k in [0, w2], with Q~[r,:] = q[i,:] * (k2[i-delta,:] + k2_bias) *
@@ -55,7 +55,9 @@ struct Cfg {
     // fills a group of RPW rows (1 KB), lane L putting the 16-byte chunk L / RPW of row
     // L % RPW at byte 16 * L.  Groups lie GROUP bytes apart.  Row operand reads and
     // transposed operand reads are both bank-conflict free in this layout.
-    static constexpr int RPW = 512 / D;                     // rows per group: 4 (D = 128) or 8 (D = 64)
+    static constexpr int RPW = 512 / D;                     // rows per group: 4 (D = 128), 8 (D = 64), 16 (D = 32)
+    // byte offset of row r of a tile (chunk 0)
+    static constexpr int row_off(int r) { return (r / RPW) * GROUP + (r % RPW) * 16; }
     static constexpr int GROUP = 1024 + 16 * RPW;           // bytes
     static constexpr int NGROUP = TJ / RPW;
     static constexpr int TILE_BYTES = NGROUP * GROUP;
@@ -190,7 +192,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
 
     // ---- workgroup accumulators ------------------------------------------------
     // thread -> (query aq, ACN columns from ac) of the fp32 accumulator in LDS
-    constexpr int ACN = D / 16;                    // columns per thread (8 or 4)
+    constexpr int ACN = D / 16;                    // columns per thread (8, 4 or 2)
     bool bad = false;
     if constexpr (!LEFT) {
         // running maximum and sum of every query: fin_m / fin_l in LDS, read and updated at the
@@ -200,15 +202,13 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
         const int io = i0 + aq < N ? i0 + aq : N - 1;
         if (has_left && !SAFE) {
             const uint16_t* prow = (const uint16_t*)p.out.p + p.out.off(b, io, h) + ac;
-            if (ACN == 8) {
-                const uint4 x = *(const uint4*)prow;
-                float* o = oacc + aq * C::OS + ac;
-                o[0] = E::lo(x.x); o[1] = E::hi(x.x); o[2] = E::lo(x.y); o[3] = E::hi(x.y);
-                o[4 % ACN] = E::lo(x.z); o[5 % ACN] = E::hi(x.z); o[6 % ACN] = E::lo(x.w); o[7 % ACN] = E::hi(x.w);
-            } else {
-                const uint2 x = *(const uint2*)prow;
-                float* o = oacc + aq * C::OS + ac;
-                o[0] = E::lo(x.x); o[1] = E::hi(x.x); o[2] = E::lo(x.y); o[3] = E::hi(x.y);
+            uint32_t pw[ACN / 2];
+            load_words(prow, pw);
+            float* o = oacc + aq * C::OS + ac;
+#pragma unroll
+            for (int c = 0; c < ACN / 2; ++c) {
+                o[2 * c] = E::lo(pw[c]);
+                o[2 * c + 1] = E::hi(pw[c]);
             }
             if (tid < BQ) {
                 const int it = i0 + tid < N ? i0 + tid : N - 1;
@@ -387,15 +387,18 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             };
             // all transposed V operand reads of a tile (opaque reads, settled before use)
             auto issue_v = [&](uint32_t vt_addr, lds_half_operand (&vh)[4 * C::DT]) {
-                lds_tr_issue<0 * DTB + 0 * (16 / C::RPW) * C::GROUP, 0 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[0], vh[1]);
-                lds_tr_issue<0 * DTB + (16 / C::RPW) * C::GROUP, 0 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[2], vh[3]);
-                lds_tr_issue<1 * DTB + 0, 1 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[4], vh[5]);
-                lds_tr_issue<1 * DTB + (16 / C::RPW) * C::GROUP, 1 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[6], vh[7]);
+                constexpr int R8 = C::row_off(8), R16 = C::row_off(16), R24 = C::row_off(24);
+                lds_tr_issue<0, R8>(vt_addr, vh[0], vh[1]);
+                lds_tr_issue<R16, R24>(vt_addr, vh[2], vh[3]);
+                if constexpr (C::DT >= 2) {
+                    lds_tr_issue<1 * DTB, 1 * DTB + R8>(vt_addr, vh[4], vh[5]);
+                    lds_tr_issue<1 * DTB + R16, 1 * DTB + R24>(vt_addr, vh[6], vh[7]);
+                }
                 if constexpr (C::DT == 4) {
-                    lds_tr_issue<2 * DTB + 0, 2 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[8], vh[9]);
-                    lds_tr_issue<2 * DTB + (16 / C::RPW) * C::GROUP, 2 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[10], vh[11]);
-                    lds_tr_issue<3 * DTB + 0, 3 * DTB + (8 / C::RPW) * C::GROUP>(vt_addr, vh[12], vh[13]);
-                    lds_tr_issue<3 * DTB + (16 / C::RPW) * C::GROUP, 3 * DTB + (24 / C::RPW) * C::GROUP>(vt_addr, vh[14], vh[15]);
+                    lds_tr_issue<2 * DTB, 2 * DTB + R8>(vt_addr, vh[8], vh[9]);
+                    lds_tr_issue<2 * DTB + R16, 2 * DTB + R24>(vt_addr, vh[10], vh[11]);
+                    lds_tr_issue<3 * DTB, 3 * DTB + R8>(vt_addr, vh[12], vh[13]);
+                    lds_tr_issue<3 * DTB + R16, 3 * DTB + R24>(vt_addr, vh[14], vh[15]);
                 }
             };
             auto value_mfmas = [&](uint32_t vt_addr, const X8* w) {
@@ -720,14 +723,12 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
 #pragma unroll
             for (int w = 1; w < FW; ++w) {
                 const uint16_t* sp = slab_of(w) + aq * C::SS + ac;
-                if (ACN == 8) {
-                    const uint4 x = *(const uint4*)sp;
-                    acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
-                    acc[4 % ACN] += bf16_lo(x.z); acc[5 % ACN] += bf16_hi(x.z);
-                    acc[6 % ACN] += bf16_lo(x.w); acc[7 % ACN] += bf16_hi(x.w);
-                } else {
-                    const uint2 x = *(const uint2*)sp;
-                    acc[0] += bf16_lo(x.x); acc[1] += bf16_hi(x.x); acc[2] += bf16_lo(x.y); acc[3] += bf16_hi(x.y);
+                uint32_t sw[ACN / 2];
+                load_words(sp, sw);
+#pragma unroll
+                for (int c = 0; c < ACN / 2; ++c) {
+                    acc[2 * c] += bf16_lo(sw[c]);
+                    acc[2 * c + 1] += bf16_hi(sw[c]);
                 }
             }
 #pragma unroll
@@ -745,11 +746,10 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
         const float Ms = fin_m[aq], L = fin_l[aq];
         const float inv = 1.f / (L + 1e-8f * fast_exp2(-Ms));
         uint16_t* orow = (uint16_t*)p.out.p + p.out.off(b, io, h) + ac;
-        union { EL h[8]; uint4 u4; uint2 u2; } o;
+        union { EL h[ACN]; uint32_t w[ACN / 2]; } o;
 #pragma unroll
         for (int c = 0; c < ACN; ++c) o.h[c] = (EL)(oacc[aq * C::OS + ac + c] * inv);
-        if (ACN == 8) *(uint4*)orow = o.u4;
-        else *(uint2*)orow = o.u2;
+        store_words(orow, o.w);
         if ((tid_f & 15) == 0) {
             float lse;
             if (Ms > LOG2_EPS) lse = LN2 * (Ms + __log2f(L + 1e-8f * fast_exp2(-Ms)));
@@ -807,7 +807,7 @@ bool aligned16(const Tensor& t, int B, int N, int H) {
 
 bool mfma_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
     (void)B; (void)H; (void)w1; (void)w2; (void)N;
-    return (dtype == SA2_BF16 || dtype == SA2_F16) && (D == 64 || D == 128);
+    return (dtype == SA2_BF16 || dtype == SA2_F16) && (D == 32 || D == 64 || D == 128);
 }
 
 bool mfma_layout_ok(const Problem& p, bool backward) {
@@ -827,8 +827,12 @@ int launch_mfma_fwd(const Problem& p, int dtype, hipStream_t st) {
     const int64_t total = (int64_t)nqb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
     if (dtype == SA2_F16)
-        return p.D == 128 ? launch_fwd_pair<ElemF16, 128>(p, nqb, (int)total, st) : launch_fwd_pair<ElemF16, 64>(p, nqb, (int)total, st);
-    return p.D == 128 ? launch_fwd_pair<ElemBF16, 128>(p, nqb, (int)total, st) : launch_fwd_pair<ElemBF16, 64>(p, nqb, (int)total, st);
+        return p.D == 128 ? launch_fwd_pair<ElemF16, 128>(p, nqb, (int)total, st)
+               : p.D == 64 ? launch_fwd_pair<ElemF16, 64>(p, nqb, (int)total, st)
+                           : launch_fwd_pair<ElemF16, 32>(p, nqb, (int)total, st);
+    return p.D == 128 ? launch_fwd_pair<ElemBF16, 128>(p, nqb, (int)total, st)
+           : p.D == 64 ? launch_fwd_pair<ElemBF16, 64>(p, nqb, (int)total, st)
+                       : launch_fwd_pair<ElemBF16, 32>(p, nqb, (int)total, st);
 }
 
 }  // namespace sa2

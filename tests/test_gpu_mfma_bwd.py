@@ -26,6 +26,8 @@ SMALL = [  # B, N, H, D, w1, w2, k2_bias, v2_bias
     (1, 33, 1, 64, 31, 32, 0.0, 0.0),
     (1, 300, 2, 128, 130, 3, 0.0, 0.0),
     (1, 1, 1, 64, 4, 4, 0.0, 0.0),
+    (2, 130, 2, 32, 33, 8, 0.1, 0.2),         # head_dim 32
+    (1, 200, 1, 32, 64, 32, 0.0, 0.0),
     (1, 200, 1, 128, 16, 150, 0.0, 0.1),     # K' window too wide for the on-chip kernels: workspace kernels
     (1, 180, 2, 128, 40, 100, 0.2, 0.0),     # K'-side on chip (q, dO rows from global memory), K-side workspace kernel
 ]

@@ -39,6 +39,8 @@ SMALL = [  # B, N, H, D, w1, w2, k2_bias, v2_bias
     (2, 160, 3, 128, 64, 32, 1.0, 0.5),
     (1, 33, 1, 64, 31, 32, 0.0, 0.0),
     (1, 1, 1, 64, 4, 4, 0.0, 0.0),
+    (2, 130, 2, 32, 33, 8, 0.1, 0.2),         # head_dim 32
+    (1, 200, 1, 32, 64, 32, 0.0, 0.0),
 ]
 
 
@@ -93,7 +95,8 @@ def test_auto_dispatch_takes_mfma_for_bf16_d64_d128():
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_BF16) == 1
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F16) == 1
     assert lib.sa2_uses_mfma(1, 128, 2, 64, 32, 16, _lib.SA2_F32) == 0
-    assert lib.sa2_uses_mfma(1, 128, 2, 32, 32, 16, _lib.SA2_BF16) == 0
+    assert lib.sa2_uses_mfma(1, 128, 2, 32, 32, 16, _lib.SA2_BF16) == 1
+    assert lib.sa2_uses_mfma(1, 128, 2, 48, 32, 16, _lib.SA2_BF16) == 0
     inp = make_inputs(1, 96, 2, 64, seed=1, dtype=torch.bfloat16, with_dout=False)
     a = fwd(inp, 20, 6, flags=0)
     b = fwd(inp, 20, 6, flags=MFMA)
