@@ -1,6 +1,6 @@
-// bf16 MFMA backward for gfx950, head_dim 64 or 128: dispatch, and the workspace kernels
-// that serve shapes whose K' window is too wide for the on-chip kernels
-// (sa2_mfma_bwd_kp.hip for dQ, dK', dV'; sa2_mfma_bwd_kv.hip for dK, dV).
+// MFMA backward for gfx950: dispatch to the on-chip kernels (sa2_mfma_bwd_kp.hip for dQ, dK',
+// dV'; sa2_mfma_bwd_kv.hip for dK, dV; bf16 or fp16, head_dim 32, 64 or 128), and the bf16
+// workspace kernels (head_dim 64 or 128) that serve shapes whose K' window is too wide for them.
 //
 // Same expanded-row view as the forward: rows r = (i, delta), Q~[r] = q[i] *
 // k2~[i-delta] * scale*log2(e) and dO~[r] = dO[i] * v2~[i-delta], both bf16.  With
