@@ -79,7 +79,7 @@ struct KpCfg {
 // four (w2 + 1 = 4n + 1).  A workgroup takes four consecutive K' blocks, one per wavefront
 // pair, and computes the unit delta = w2 of each in one shared sweep of K/V tiles.  Its
 // results go where the main kernel (launched next with left = 1) picks them up: dK'
-// (unscaled) and dV' in the element type in the output tensors, the dQ contribution as fp32 in rows
+// and dV' in the element type in the output tensors, the dQ contribution as fp32 in rows
 // w2 .. w2+31 of the block's dQ partial.  The main kernel then handles delta < w2.
 template <class E, int D, bool RAW, bool LEFT>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -290,25 +290,8 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) pacc[dt][v] = 0.f;
-    // the first pair starts from the pre-pass results (dK' is scaled at the end)
-    auto start_from = [&](const Tensor& t) {
-        if (!(has_left && pr == 0 && t.p)) return;
-        const int tid_i = kp_recompute_here(threadIdx.x);
-        const int k = k0 + (tid_i & 31) < N ? k0 + (tid_i & 31) : N - 1;
-        const uint16_t* src = (const uint16_t*)t.p + t.off(b, k, h) + 4 * ((tid_i >> 5) & 1);
-#pragma unroll
-        for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const uint2 x = *(const uint2*)(src + dt * 32 + 8 * g4);
-                pacc[dt][4 * g4 + 0] = E::lo(x.x); pacc[dt][4 * g4 + 1] = E::hi(x.x);
-                pacc[dt][4 * g4 + 2] = E::lo(x.y); pacc[dt][4 * g4 + 3] = E::hi(x.y);
-            }
-    };
-
     if (role == 0) {
         // =============================== P wavefronts ================================
-        start_from(p.dv2);
         for (int round = 0; round < nrounds; ++round) {
             const int delta = LEFT ? w2 : round * NPAIR + pr;
             const bool ok = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta < n_units;
@@ -446,7 +429,6 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         }
     } else {
         // =============================== dS wavefronts ===============================
-        start_from(p.dk2);
         for (int round = 0; round < nrounds; ++round) {
             const int delta = LEFT ? w2 : round * NPAIR + pr;
             const bool ok = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta < n_units;
@@ -548,7 +530,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                     }
             }
             if constexpr (LEFT) {
-                // pre-pass: dK' of the unit (unscaled) goes to the output tensor, its dQ
+                // pre-pass: dK' of the unit goes to the output tensor, its dQ
                 // contribution G * k2~ (unscaled) to rows w2 .. w2+31 of the block's dQ partial
                 if (ok && k0 + ln < N) {
                     if (p.dk2.p) {
@@ -559,7 +541,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                             for (int g4 = 0; g4 < 4; ++g4) {
                                 union { EL hh[4]; uint2 u; } o;
 #pragma unroll
-                                for (int x = 0; x < 4; ++x) o.hh[x] = (EL)pacc[dt][4 * g4 + x];
+                                for (int x = 0; x < 4; ++x) o.hh[x] = (EL)(p.scale * pacc[dt][4 * g4 + x]);
                                 *(uint2*)(dst + dt * 32 + 8 * g4) = o.u;
                             }
                     }
@@ -662,6 +644,24 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     }
     __syncthreads();
     // ---- dK' and dV': add the four wavefronts of each role through LDS ----------------
+    // item -> (tensor, K' row, 8 columns); a thread's items are it = tid, tid + KT, ...
+    constexpr int CHF = D / 8;
+    constexpr int ITEMS = (2 * BQ * CHF + KT - 1) / KT;
+    // what the pre-pass left in the output rows (the contribution of the unit delta = w2),
+    // requested now so that it arrives while the wavefronts' sums go through LDS
+    uint4 pre[ITEMS];
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        pre[j] = make_uint4(0, 0, 0, 0);
+        const int it = tid_f + j * KT;
+        if (it < 2 * BQ * CHF && has_left) {
+            const int which = it / (BQ * CHF);
+            const int rem = it - which * BQ * CHF;
+            const int row = rem / CHF, c0 = (rem - row * CHF) * 8;
+            const Tensor& t = which ? p.dk2 : p.dv2;
+            if (k0 + row < N && t.p) pre[j] = *(const uint4*)((const uint16_t*)t.p + t.off(b, k0 + row, h) + c0);
+        }
+    }
     {
         float* region = (float*)smem_raw + (size_t)wave * BQ * C::AS;
         const int ln_f = tid_f & 31, hf_f = (tid_f >> 5) & 1;
@@ -678,9 +678,12 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     }
     __syncthreads();
     {
-        constexpr int CH = D / 8;
+        constexpr int CH = CHF;
         const float* base = (const float*)smem_raw;
-        for (int it = tid_f; it < 2 * BQ * CH; it += KT) {
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int it = tid_f + j * KT;
+            if (it >= 2 * BQ * CH) break;
             const int which = it / (BQ * CH);                       // 0: dV' (P wavefronts), 1: dK'
             const int rem = it - which * BQ * CH;
             const int row = rem / CH, c0 = (rem - row * CH) * 8;
@@ -698,10 +701,14 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
             }
             const float sc = which ? p.scale : 1.f;
+            uint16_t* dst = (uint16_t*)t.p + t.off(b, k, h) + c0;
+            const uint4 x = pre[j];                                 // zeros where the pre-pass did not run
+            const float part[8] = {E::lo(x.x), E::hi(x.x), E::lo(x.y), E::hi(x.y),
+                                   E::lo(x.z), E::hi(x.z), E::lo(x.w), E::hi(x.w)};
             union { EL hh[8]; uint4 u; } o;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) o.hh[c] = (EL)(acc[c] * sc);
-            *(uint4*)((uint16_t*)t.p + t.off(b, k, h) + c0) = o.u;
+            for (int c = 0; c < 8; ++c) o.hh[c] = (EL)(acc[c] * sc + part[c]);
+            *(uint4*)dst = o.u;
         }
     }
 }
