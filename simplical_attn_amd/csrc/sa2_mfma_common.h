@@ -174,6 +174,36 @@ template <class X8 = bf16x8>
 __device__ __forceinline__ X8 lds_read_x8(uint32_t addr) {
     return *(const X8 __attribute__((address_space(3)))*)(uintptr_t)addr;
 }
+// Row operand reads as opaque instructions, like lds_tr_issue: r[FIRST + i] = the 16 bytes at
+// addr + (FIRST + i) * STEP for i < N.  The compiler's own wait-count bookkeeping does not see
+// them (nor the transposed reads), so it neither waits for them nor makes a wait for one of its
+// own loads cover them; lds_wait<PENDING>() names the registers that may be used once at most
+// PENDING of the LDS reads issued so far are still outstanding (they return in order).
+template <int FIRST, int N, int STEP, class X8>
+__device__ __forceinline__ void lds_row_issue(uint32_t addr, X8* r) {
+    if constexpr (N > 0) {
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r[FIRST]) : "v"(addr), "n"(FIRST * STEP));
+        lds_row_issue<FIRST + 1, N - 1, STEP>(addr, r);
+    }
+}
+template <int PENDING, class X8>
+__device__ __forceinline__ void lds_wait(X8 (&x)[1]) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x[0]) : "n"(PENDING));
+}
+template <int PENDING, class X8>
+__device__ __forceinline__ void lds_wait(X8 (&x)[2]) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x[0]), "+v"(x[1]) : "n"(PENDING));
+}
+template <int PENDING, class X8>
+__device__ __forceinline__ void lds_wait(X8 (&x)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]) : "n"(PENDING));
+}
+template <int PENDING, class X8>
+__device__ __forceinline__ void lds_wait(X8 (&x)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(%8)"
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+                 : "n"(PENDING));
+}
 
 }  // namespace
 }  // namespace sa2

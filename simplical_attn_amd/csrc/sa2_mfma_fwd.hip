@@ -166,19 +166,22 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
     const int t_row = wave * C::RPW + (lane % C::RPW), t_col = lane / C::RPW;
     const uint32_t k_off = ((uint32_t)t_row * (uint32_t)p.k1.sn + t_col * 8) * 2u;
     const uint32_t v_off = ((uint32_t)t_row * (uint32_t)p.v1.sn + t_col * 8) * 2u;
+    // the same for the tile that holds the end of the sequence: rows past it are clamped to the
+    // last one (they are masked later)
+    const int jt_end = (N - 1) / TJ;
+    const int t_row_c = t_row < N - 1 - jt_end * TJ ? t_row : N - 1 - jt_end * TJ;
+    const uint32_t k_off_c = ((uint32_t)t_row_c * (uint32_t)p.k1.sn + t_col * 8) * 2u;
+    const uint32_t v_off_c = ((uint32_t)t_row_c * (uint32_t)p.v1.sn + t_col * 8) * 2u;
     typedef __attribute__((address_space(3))) void* lds_ptr;
     typedef const __attribute__((address_space(1))) void* glb_ptr;
     int dma_tile = 0, dma_stage = 0, dma_count = 0;             // next tile (from jt_lo), its stage, tiles requested
+    // (no branch in here when every wavefront owns a group, so that the request can be scheduled
+    // into the middle of a step's arithmetic)
     auto dma_next = [&]() {
         const int j0 = (jt_lo + dma_tile) * TJ;
-        if (t_owner) {
-            uint32_t ko = k_off, vo = v_off;
-            if (__builtin_expect(j0 + TJ > N, 0)) {
-                // last tile of the sequence: clamp the rows (they are masked later)
-                const int r = t_row < N - 1 - j0 ? t_row : N - 1 - j0;
-                ko = ((uint32_t)r * (uint32_t)p.k1.sn + t_col * 8) * 2u;
-                vo = ((uint32_t)r * (uint32_t)p.v1.sn + t_col * 8) * 2u;
-            }
+        if (C::NGROUP >= FW || t_owner) {
+            const bool at_end = jt_lo + dma_tile == jt_end;
+            const uint32_t ko = at_end ? k_off_c : k_off, vo = at_end ? v_off_c : v_off;
             const char* kb = (const char*)(k1p + (int64_t)j0 * p.k1.sn);
             const char* vb = (const char*)(v1p + (int64_t)j0 * p.v1.sn);
             unsigned char* dst = smem_raw + (size_t)dma_stage * (C::STAGE * 2) + wave * C::GROUP;
@@ -511,20 +514,21 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 uint32_t vt_prev = stage_addr(buf) + (uint32_t)C::TILE_BYTES + v_lane;
                 advance();
                 // One step: logits of tile s into `cur`, weights and value MFMAs of tile s-1 from `prev`.
-                auto step = [&](int s, const floatx16& prev, floatx16& cur) {
-                    begin_step(s);
+                // PLAIN: the tile needs no mask.  DMA: the step requests a tile (all but the last
+                // two steps of the kernel do).  Both are compile-time so that a step is one
+                // basic block: the request's scalar arithmetic and the loads then sit between the
+                // MFMAs instead of in front of them, where both wavefronts of a SIMD would wait.
+                auto step = [&](int s, const floatx16& prev, floatx16& cur, auto PLAIN_TAG, auto DMA_TAG) {
+                    constexpr bool PLAIN = decltype(PLAIN_TAG)::value, DMA = decltype(DMA_TAG)::value;
                     const uint32_t ks_addr = stage_addr(buf);
                     X8 ka[C::DK];
 #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_x8<X8>(ks_addr + k_lane + kk * KKB);
-                    // the reference point (and, on the two window-edge tiles, the mask) is the
+                    // the reference point (and, on the window-edge tiles, the mask) is the
                     // C operand of the first logit MFMA
-                    if (__builtin_expect(tile_plain(s), 1)) {
-                        cur = E::mfma(ka[0], qf[0], negm, 0, 0, 0);
-                    } else {
-                        asm volatile("" ::: "memory");      // keep the mask arithmetic out of the common path
-                        cur = E::mfma(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
-                    }
+                    if constexpr (PLAIN) cur = E::mfma(ka[0], qf[0], negm, 0, 0, 0);
+                    else cur = E::mfma(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
+                    if constexpr (DMA) dma_next();
                     lds_half_operand vh[4 * C::DT];
                     issue_v(vt_prev, vh);
                     X8 pb[2];
@@ -535,38 +539,64 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     weights(prev, pb, rs);
                     l += rs;
                     bad |= !(rs < E::WEIGHT_LIMIT);
+                    asm volatile("" : "+v"(pb[0]));
                     lds_settle(vh);
 #pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
+                    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                        for (int ks = 0; ks < 2; ++ks) {
+                        for (int dt = 0; dt < C::DT; ++dt) {
                             const X8 va = lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
                             racc[dt] = E::mfma(va, pb[ks], racc[dt], 0, 0, 0);
                         }
+                    // the softmax arithmetic is spread over all MFMAs of the step: the first half of
+                    // the weights under the logit MFMAs, the second half under the first half's
+                    // value MFMAs, the row sum under the rest
+                    constexpr int PER = (36 + C::DK + 2 * C::DT - 1) / (C::DK + 2 * C::DT);
 #pragma unroll
-                    for (int x = 1; x < C::DK; ++x) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one logit MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x402, 5, 0);               // a slice of VALU / exp
+                    for (int x = 0; x < C::DK + 2 * C::DT; ++x) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x402, PER, 0);             // a slice of VALU / exp
                     }
                     vt_prev = ks_addr + (uint32_t)C::TILE_BYTES + v_lane;
-                    advance();
+                    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    buf = (buf + 1) & (C::NSTAGE - 1);
+                    ++g;
                 };
+                // Steps s .. to of one kind; sh_a holds the shifted logits of the latest tile before
+                // and after.  The steps that still request a tile come first.
                 int s = ws0 + 1;
-                for (; s + 1 <= ws1; s += 2) {
-                    step(s, sh_a, sh_b);
-                    step(s + 1, sh_b, sh_a);
+                auto run = [&](int to, auto PLAIN_TAG) {
+                    const int left_to_request = total_steps - dma_count;
+                    const int to_dma = to - s + 1 <= left_to_request ? to : s + left_to_request - 1;
+                    for (; s + 1 <= to_dma; s += 2) {
+                        step(s, sh_a, sh_b, PLAIN_TAG, std::true_type{});
+                        step(s + 1, sh_b, sh_a, PLAIN_TAG, std::true_type{});
+                    }
+                    if (s <= to_dma) {
+                        step(s, sh_a, sh_b, PLAIN_TAG, std::true_type{});
+                        sh_a = sh_b;
+                        ++s;
+                    }
+                    for (; s <= to; ++s) {               // the last two steps of the kernel
+                        step(s, sh_a, sh_b, std::false_type{}, std::false_type{});
+                        sh_a = sh_b;
+                    }
+                };
+                // window-edge tiles, tiles that need no mask, window-edge tiles
+                const int p_lo = rows_full ? (s_lo > s ? s_lo : s) : ws1 + 1;
+                const int p_hi = rows_full ? (s_hi < ws1 ? s_hi : ws1) : ws1;
+                if (p_lo <= p_hi) {
+                    run(p_lo - 1, std::false_type{});
+                    run(p_hi, std::true_type{});
                 }
+                run(ws1, std::false_type{});
                 X8 pb[2];
                 float rs;
-                if (s <= ws1) {
-                    step(s, sh_a, sh_b);
-                    weights(sh_b, pb, rs);
-                } else {
-                    weights(sh_a, pb, rs);
-                }
+                weights(sh_a, pb, rs);
                 l += rs;
                 bad |= !(rs < E::WEIGHT_LIMIT);
-                value_mfmas(vt_prev - v_lane + v_lane, pb);
+                value_mfmas(vt_prev, pb);
                 for (int s2 = ws1 + 1; s2 < nt; ++s2) {   // (pre-pass) tiles after this wavefront's window
                     begin_step(s2);
                     advance();
