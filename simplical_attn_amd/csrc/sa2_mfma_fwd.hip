@@ -17,10 +17,12 @@
 // four-stage LDS ring (global_load_lds, two steps ahead of their use) in a grouped
 // layout that both the 16-byte K operand reads and the transposed V operand reads
 // (ds_read_b64_tr_b16) take without bank conflicts.  The q rows of the block and the
-// K'/V' rows its deltas reach are copied to LDS once.  On unmasked tiles each step
-// issues the logit MFMAs of tile t between the softmax instructions of tile t-1
-// and then the value MFMAs of tile t-1, so neither pipe waits for the other inside
-// the one barrier interval per tile.  After each round of 8 units the wavefronts fold their
+// K'/V' rows its deltas reach are copied to LDS once.  A step issues the logit MFMAs
+// of tile t between the softmax instructions of tile t-1, then the step's barrier (every
+// LDS read of the step is complete by then), then the value MFMAs of tile t-1, which
+// only read registers and so run under the next step's tile request and operand reads.
+// A step is one basic block (mask and request are compile-time variants of it), so that
+// the compiler can place all of this between the MFMAs.  After each round of 8 units the wavefronts fold their
 // (m, l, R*v2) into the workgroup's fp32 accumulator through bf16 slabs in LDS,
 // each thread summing a fixed slice in a fixed order.
 //
@@ -539,8 +541,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     weights(prev, pb, rs);
                     l += rs;
                     bad |= !(rs < E::WEIGHT_LIMIT);
-                    asm volatile("" : "+v"(pb[0]));
+                    asm volatile("" : "+v"(pb[0]));              // (the wait below stays behind the first weights)
                     lds_settle(vh);
+                    // The barrier stands in front of the value MFMAs: they only read registers.
+                    vt_prev = ks_addr + (uint32_t)C::TILE_BYTES + v_lane;
+                    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    buf = (buf + 1) & (C::NSTAGE - 1);
+                    ++g;
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
@@ -548,20 +556,13 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                             const X8 va = lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
                             racc[dt] = E::mfma(va, pb[ks], racc[dt], 0, 0, 0);
                         }
-                    // the softmax arithmetic is spread over all MFMAs of the step: the first half of
-                    // the weights under the logit MFMAs, the second half under the first half's
-                    // value MFMAs, the row sum under the rest
+                    // the softmax arithmetic is spread over the MFMAs of the step
                     constexpr int PER = (36 + C::DK + 2 * C::DT - 1) / (C::DK + 2 * C::DT);
 #pragma unroll
                     for (int x = 0; x < C::DK + 2 * C::DT; ++x) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
                         __builtin_amdgcn_sched_group_barrier(0x402, PER, 0);             // a slice of VALU / exp
                     }
-                    vt_prev = ks_addr + (uint32_t)C::TILE_BYTES + v_lane;
-                    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    buf = (buf + 1) & (C::NSTAGE - 1);
-                    ++g;
                 };
                 // Steps s .. to of one kind; sh_a holds the shifted logits of the latest tile before
                 // and after.  The steps that still request a tile come first.
