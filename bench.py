@@ -44,9 +44,9 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters on a plain copy kernel; None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 861.8e6,                # pre-pass 417.3 MB + fast kernel 443.4 MB + repair launch 1.1 MB
-    ("c4", "backward_k_side"): 650.0e6,        # mfma_bwd_kv_kernel
-    ("c4", "backward_kprime_side"): 1955.2e6,  # pre-pass 766.6 MB + mfma_bwd_kp_kernel 887.1 MB + dq_sum 301.5 MB
+    ("c4", "forward"): 864.2e6,                # pre-pass 419.7 MB + fast kernel 443.4 MB + repair launch 1.1 MB
+    ("c4", "backward_k_side"): 632.2e6,        # mfma_bwd_kv_kernel
+    ("c4", "backward_kprime_side"): 1954.0e6,  # pre-pass 766.5 MB + mfma_bwd_kp_kernel 886.0 MB + dq_sum 301.5 MB
 }
 
 
