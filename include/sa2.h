@@ -4,8 +4,9 @@
  * Plain C: pointers, sizes and scalars only; no torch types.  Every pointer
  * is a DEVICE pointer unless stated otherwise.  All entry points are
  * asynchronous on the HIP stream they are given, allocate nothing, never
- * synchronise, keep no state between calls and return 0 on success or a
- * negative sa2_status on error (nothing is launched on error).
+ * synchronise, keep no state that depends on a call's arguments (each kernel's
+ * LDS limit is raised once per process and device) and return 0 on success or
+ * a negative sa2_status on error (nothing is launched on error).
  *
  * Tensors are [B, N, H, D] with per-tensor ELEMENT strides (batch, sequence,
  * head); the D stride must be 1.  LSE and workspace rows are [B, H, N] fp32,

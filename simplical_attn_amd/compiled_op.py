@@ -21,8 +21,9 @@ def forward_op(q: Tensor, k1: Tensor, k2: Tensor, v1: Tensor, v2: Tensor, w1: in
 
 @forward_op.register_fake
 def _(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias):
-    B, N, H, _ = q.shape
-    return torch.empty_like(q), q.new_empty((B, H, N), dtype=torch.float32)
+    # the real op returns freshly allocated contiguous tensors whatever the strides of q
+    B, N, H, D = q.shape
+    return q.new_empty((B, N, H, D)), q.new_empty((B, H, N), dtype=torch.float32)
 
 
 @torch.library.custom_op("simplical_attn_amd::backward", mutates_args=())
@@ -34,7 +35,7 @@ def backward_op(q: Tensor, k1: Tensor, k2: Tensor, v1: Tensor, v2: Tensor, out: 
 
 @backward_op.register_fake
 def _(q, k1, k2, v1, v2, out, lse, dout, w1, w2, scale, k2_bias, v2_bias):
-    return tuple(torch.empty_like(t) for t in (q, k1, k2, v1, v2))
+    return tuple(t.new_empty(tuple(t.shape)) for t in (q, k1, k2, v1, v2))
 
 
 def _setup_context(ctx, inputs, output):

@@ -1,10 +1,36 @@
 // extern "C" boundary: argument validation and kernel-path selection.
-// No allocation, no synchronisation, no global state.
+// No allocation and no synchronisation.  The only process state is set-up that happens once and
+// never depends on a call's arguments: each kernel's LDS limit (allow_full_lds).
 #include <string.h>
+
+#include <mutex>
+#include <utility>
+#include <vector>
 
 #include "sa2_common.h"
 
 using namespace sa2;
+
+namespace sa2 {
+
+bool allow_full_lds(const void* kernel) {
+    static std::mutex mu;
+    static std::vector<std::pair<const void*, int>> done;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    std::lock_guard<std::mutex> lock(mu);
+    for (const auto& e : done)
+        if (e.first == kernel && e.second == dev) return true;
+    // the limit covers dynamic LDS only: what the kernel declares statically comes off the 160 KB
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, kernel) != hipSuccess) return false;
+    const int room = LDS_BYTES_PER_CU - (int)attr.sharedSizeBytes;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, room) != hipSuccess) return false;
+    done.emplace_back(kernel, dev);
+    return true;
+}
+
+}  // namespace sa2
 
 namespace {
 
@@ -44,8 +70,6 @@ bool strides_ok(const int64_t* strides, int count, int B, int N, int H) {
 }
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
-
-size_t dsum_bytes(int B, int N, int H) { return align_up((size_t)B * H * N * sizeof(float), 256); }
 
 bool pick_mfma(const Problem& p, int dtype, unsigned flags, bool backward, int* status) {
     *status = SA2_OK;

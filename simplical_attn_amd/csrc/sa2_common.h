@@ -66,6 +66,12 @@ __device__ __forceinline__ float lse_with_eps(float m, float l) {
     return log_eps + log1pf(l * expf(m - log_eps));
 }
 
+// Lifts a kernel's limit on dynamic LDS to the CU's full 160 KB.  The value never depends on the
+// call, and it is set once per (kernel, device) for the life of the process, so concurrent
+// launches of one kernel with different LDS sizes cannot disturb each other.
+constexpr int LDS_BYTES_PER_CU = 160 * 1024;
+bool allow_full_lds(const void* kernel);
+
 // ---- launchers (each returns a sa2_status) ----------------------------------
 int launch_rowdot(const Tensor& out, const Tensor& dout, float* dsum, int B, int N, int H, int D,
                   int dtype, hipStream_t st);

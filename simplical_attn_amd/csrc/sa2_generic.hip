@@ -377,8 +377,7 @@ int check_launch() { return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_L
 
 template <typename K>
 bool allow_big_lds(K kernel, size_t bytes) {
-    return bytes <= 64 * 1024 ||
-           hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess;
+    return bytes <= 64 * 1024 || allow_full_lds((const void*)kernel);
 }
 
 }  // namespace

@@ -579,9 +579,7 @@ int launch_col_part(const Problem& p, hipStream_t st) {
     const int njb = (p.N + CJ - 1) / CJ;
     const int64_t total = (int64_t)njb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-    if (hipFuncSetAttribute((const void*)mfma_bwd_col_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)C::LDS_BYTES) != hipSuccess)
-        return SA2_ERR_LAUNCH_FAILED;
+    if (!allow_full_lds((const void*)mfma_bwd_col_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
     hipLaunchKernelGGL(mfma_bwd_col_kernel<D>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, njb,
                        (int)total);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
@@ -601,9 +599,7 @@ int launch_row_part(const Problem& p, hipStream_t st) {
     if (p.scratch_bytes < 2 * one) return SA2_ERR_WORKSPACE_TOO_SMALL;
     uint16_t* gws = (uint16_t*)p.scratch;
     uint16_t* rws = (uint16_t*)((char*)p.scratch + one);
-    if (hipFuncSetAttribute((const void*)mfma_bwd_row_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)C::LDS_BYTES) != hipSuccess)
-        return SA2_ERR_LAUNCH_FAILED;
+    if (!allow_full_lds((const void*)mfma_bwd_row_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
     hipLaunchKernelGGL(mfma_bwd_row_kernel<D>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, nqb,
                        (int)total, gws, rws);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;

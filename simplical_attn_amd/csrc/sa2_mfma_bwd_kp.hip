@@ -762,16 +762,13 @@ int launch_kp(const Problem& p, hipStream_t st) {
         const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + C::PX_BYTES;
         const int ngrp = (nkb + NPAIR - 1) / NPAIR;
         const int64_t total_left = (int64_t)ngrp * p.B * p.H;
-        if (hipFuncSetAttribute((const void*)mfma_bwd_kp_kernel<E, D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_left) != hipSuccess)
-            return SA2_ERR_LAUNCH_FAILED;
+        if (!allow_full_lds((const void*)mfma_bwd_kp_kernel<E, D, false, true>)) return SA2_ERR_LAUNCH_FAILED;
         hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, true>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
                            (int)total_left, part, 0);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
     const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<E, D, true, false> : (const void*)mfma_bwd_kp_kernel<E, D, false, false>;
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return SA2_ERR_LAUNCH_FAILED;
+    if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
     if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, true, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
     else hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;

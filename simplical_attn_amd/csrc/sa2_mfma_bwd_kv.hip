@@ -366,8 +366,7 @@ int launch_kv(const Problem& p, hipStream_t st) {
     const size_t lds = C::lds_bytes(p.w2);
     const bool bias = p.k2_bias != 0.f || p.v2_bias != 0.f;
     const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<E, D, true> : (const void*)mfma_bwd_kv_kernel<E, D, false>;
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return SA2_ERR_LAUNCH_FAILED;
+    if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
     if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
     else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;

@@ -797,12 +797,9 @@ int launch_fwd_kernels(const Problem& p, int nqb, int total, hipStream_t st) {
     // one unit left over after the rounds of eight: the pre-pass takes it, unless the grid is so
     // small that a further launch costs more than the lone round
     const int left = (p.w2 >= FW && p.w2 % FW == 0 && (p.force_prepass || total >= PREPASS_MIN_WORKGROUPS)) ? 1 : 0;
-    if (hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_FAST, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess ||
-        hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_SAFE, SIDE>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess ||
-        hipFuncSetAttribute((const void*)mfma_fwd_kernel<E, D, MODE_LEFT, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)C::STAGE_BYTES) != hipSuccess)
+    if (!allow_full_lds((const void*)mfma_fwd_kernel<E, D, MODE_FAST, SIDE>) ||
+        !allow_full_lds((const void*)mfma_fwd_kernel<E, D, MODE_SAFE, SIDE>) ||
+        !allow_full_lds((const void*)mfma_fwd_kernel<E, D, MODE_LEFT, false>))
         return SA2_ERR_LAUNCH_FAILED;
     if (left) {
         const int ngrp = (nqb + FW - 1) / FW;

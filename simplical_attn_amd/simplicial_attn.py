@@ -36,8 +36,12 @@ def _check_inputs(q, k1, k2, v1, v2):
 
 
 def _rows(t):
-    """Tensor usable by the kernels: unit stride along head_dim."""
-    return t if t.stride(-1) == 1 else t.contiguous()
+    """Tensor usable by the kernels: unit stride along head_dim and a positive stride on every
+    axis longer than 1.  Broadcast views (stride 0: a gradient expanded by ``sum`` in the loss,
+    a key expanded over heads) and anything else are copied, as the reference's launch accepts
+    arbitrary strides (simplicial/triton_impl.py:38-45)."""
+    ok = t.stride(-1) == 1 and all(st > 0 or n == 1 for st, n in zip(t.stride()[:-1], t.shape[:-1]))
+    return t if ok else t.contiguous()
 
 
 def _strides(*tensors):
@@ -103,9 +107,9 @@ def simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2, scale=None, k
     return tuple(grads)
 
 
-def compute_D_kernel(dO, O):
-    """sum_d dO*O per (batch, head, position) in fp32, [B,H,N].  Same job as the
-    reference helper of that name (simplicial/kernels.py:569-571)."""
+def simplicial_rowdot(dO, O):
+    """sum_d dO*O per (batch, head, position) in fp32, laid out [B,H,N] as the backward
+    kernels index it (C entry point sa2_rowdot)."""
     lib = _lib.load()
     B, N, H, D = O.shape
     O, dO = _rows(O), _rows(dO)
@@ -114,6 +118,12 @@ def compute_D_kernel(dO, O):
         _lib.check(lib.sa2_rowdot(O.data_ptr(), dO.data_ptr(), dsum.data_ptr(), B, N, H, D,
                                   _strides(O, dO), _DTYPES[O.dtype], _stream(O)))
     return dsum
+
+
+def compute_D_kernel(dO, O):
+    """The reference helper of that name (simplicial/kernels.py:569-571): ``sum(dO * O, dim=-1)``,
+    shape [B,N,H] in dO's dtype.  The sum itself is taken in fp32 by the device kernel."""
+    return simplicial_rowdot(dO, O).transpose(1, 2).to(dO.dtype)
 
 
 class TwoSimplicialAttentionFunction(torch.autograd.Function):
@@ -169,16 +179,18 @@ class _ExactFunction(torch.autograd.Function):
         return (*grads, None, None, None, None, None)
 
 
-def two_simplicial_attention_reference(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0):
-    """Signature of the reference's PyTorch implementation (simplicial/reference.py:8-9).  Here it
-    runs the fp32 FMA kernels on the GPU (same windows, bias and epsilon as reference.py:27-76) and
-    is differentiable; it is the device-side yardstick for the MFMA kernels, not a CPU path."""
+def two_simplicial_attention_exact(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0):
+    """Argument list of the reference's PyTorch implementation (simplicial/reference.py:8-9), run
+    on the fp32 FMA kernels on the GPU (same windows, bias and epsilon as reference.py:27-76),
+    differentiable.  It is a device-side yardstick for the MFMA kernels: HIP kernels of this same
+    library, NOT an independent reference and not a CPU path.  Comparing the operator with it is a
+    kernel-against-kernel check."""
     return _ExactFunction.apply(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias)
 
 
-class TwoSimplicialAttentionReference(torch.nn.Module):
-    """Module wrapper of two_simplicial_attention_reference with the reference's constructor
-    (simplicial/reference.py:79-103)."""
+class TwoSimplicialAttentionExact(torch.nn.Module):
+    """Module wrapper of two_simplicial_attention_exact with the constructor of the reference's
+    TwoSimplicialAttentionReference (simplicial/reference.py:79-103)."""
 
     def __init__(self, head_dim, w1=64, w2=64, scale=None, k2_bias=0.0, v2_bias=0.0):
         super().__init__()
@@ -190,8 +202,8 @@ class TwoSimplicialAttentionReference(torch.nn.Module):
         self.v2_bias = v2_bias
 
     def forward(self, q, k1, k2, v1, v2):
-        return two_simplicial_attention_reference(q, k1, k2, v1, v2, self.w1, self.w2, self.scale,
-                                                  self.k2_bias, self.v2_bias)
+        return two_simplicial_attention_exact(q, k1, k2, v1, v2, self.w1, self.w2, self.scale,
+                                              self.k2_bias, self.v2_bias)
 
 
 class TwoSimplicialAttention(torch.nn.Module):

@@ -90,12 +90,16 @@ def test_reference_package_names():
     """Every name the reference package exports (simplicial/__init__.py:12-27) either exists with the
     reference's signature or raises an AttributeError that says what to use instead."""
     import simplical_attn_amd as sa
-    rsig = inspect.signature(sa.two_simplicial_attention_reference)
+    rsig = inspect.signature(sa.two_simplicial_attention_exact)
     assert list(rsig.parameters) == ["q", "k1", "k2", "v1", "v2", "w1", "w2", "scale", "k2_bias", "v2_bias"]
     assert [rsig.parameters[k].default for k in ("scale", "k2_bias", "v2_bias")] == [None, 0.0, 0.0]
-    m = sa.TwoSimplicialAttentionReference(16, 4, 4)
+    m = sa.TwoSimplicialAttentionExact(16, 4, 4)
     assert m.scale == 0.25 and list(inspect.signature(m.forward).parameters) == ["q", "k1", "k2", "v1", "v2"]
     assert callable(sa.compute_D_kernel)
+    # the device yardstick does not pose as the reference's CPU loop
+    for name in ("two_simplicial_attention_reference", "TwoSimplicialAttentionReference"):
+        with pytest.raises(AttributeError, match="kernel-against-kernel"):
+            getattr(sa, name)
     for name in ("two_simplicial_attn_fwd_kernel", "two_simplicial_attn_bwd_kv1_kernel",
                  "two_simplicial_attn_bwd_kv2_kernel", "run_all_correctness_tests", "run_all_performance_tests",
                  "quick_performance_test", "run_all_tests", "test_forward_pass_correctness",
@@ -104,7 +108,7 @@ def test_reference_package_names():
             getattr(sa, name)
     x = torch.zeros(1, 8, 1, 16)
     with pytest.raises(RuntimeError, match="GPU only"):
-        sa.two_simplicial_attention_reference(x, x, x, x, x, 4, 4)
+        sa.two_simplicial_attention_exact(x, x, x, x, x, 4, 4)
 
 
 def test_cpu_tensors_fail_loudly():

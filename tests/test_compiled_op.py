@@ -17,6 +17,20 @@ def test_fake_implementations_give_shapes_and_dtypes():
     assert len(grads) == 5 and all(g.shape == (B, N, H, D) and g.dtype == torch.bfloat16 for g in grads)
 
 
+def test_fake_outputs_are_contiguous_like_the_real_ones():
+    """The kernels' results are freshly allocated contiguous tensors whatever the strides of the
+    inputs; the fake implementations must say the same or compiled graphs mis-address them."""
+    B, N, H, D = 2, 40, 3, 64
+    x = [torch.empty(B, H, N, D, dtype=torch.bfloat16, device="meta").transpose(1, 2) for _ in range(6)]
+    assert not x[0].is_contiguous()
+    out, lse = forward_op(*x[:5], 8, 4, 0.125, 0.0, 0.0)
+    want = torch.empty(B, N, H, D, device="meta").stride()
+    assert out.shape == (B, N, H, D) and out.stride() == want
+    assert lse.stride() == torch.empty(B, H, N, device="meta").stride()
+    grads = backward_op(*x[:5], out, lse, x[5], 8, 4, 0.125, 0.0, 0.0)
+    assert all(g.shape == (B, N, H, D) and g.stride() == want for g in grads)
+
+
 @pytest.mark.gpu
 def test_traced_op_matches_the_eager_function():
     dev = torch.device("cuda:0")

@@ -191,15 +191,15 @@ def test_error_codes():
         simplicial_forward(y.cpu(), y.cpu(), y.cpu(), y.cpu(), y.cpu(), 4, 4)
 
 
-def test_reference_named_entry_points_run_the_exact_kernels():
-    """two_simplicial_attention_reference / TwoSimplicialAttentionReference (the reference's names,
+def test_exact_entry_points_run_the_fp32_kernels():
+    """two_simplicial_attention_exact / TwoSimplicialAttentionExact (argument lists of
     simplicial/reference.py:8, 79): bf16 tensors, fp32 arithmetic, differentiable; they agree with
     the oracle more closely than the bf16 parity bar and with the MFMA kernels within it."""
     import simplical_attn_amd as sa
     dev = torch.device("cuda:0")
     inp = make_inputs(1, 96, 2, 64, seed=9, dtype=torch.bfloat16)
     leaves = [x.to(dev).requires_grad_(True) for x in inp[:5]]
-    out = sa.TwoSimplicialAttentionReference(64, 20, 6, k2_bias=0.1)(*leaves)
+    out = sa.TwoSimplicialAttentionExact(64, 20, 6, k2_bias=0.1)(*leaves)
     out.backward(inp[5].to(dev))
     want = oracle_all(inp, 20, 6, None, 0.1, 0.0)
     assert_close_rel(out, want["out"], 5e-3, "out")
@@ -210,9 +210,50 @@ def test_reference_named_entry_points_run_the_exact_kernels():
 
 
 def test_rowdot():
-    from simplical_attn_amd import compute_D_kernel
+    from simplical_attn_amd import compute_D_kernel, simplicial_rowdot
     dev = torch.device("cuda:0")
     a = torch.randn(2, 33, 3, 40, device=dev, dtype=torch.bfloat16)
     b = torch.randn(2, 33, 3, 40, device=dev, dtype=torch.bfloat16)
-    want = (a.float() * b.float()).sum(-1).permute(0, 2, 1)
-    assert torch.allclose(compute_D_kernel(a, b), want, rtol=1e-5, atol=1e-5)
+    want = (a.float() * b.float()).sum(-1)                           # [B,N,H]
+    assert torch.allclose(simplicial_rowdot(a, b), want.permute(0, 2, 1), rtol=1e-5, atol=1e-5)
+    # the reference helper's layout and dtype (simplicial/kernels.py:569-571): [B,N,H] like dO
+    got = compute_D_kernel(a, b)
+    assert got.shape == (2, 33, 3) and got.dtype == torch.bfloat16
+    assert torch.equal(got, want.to(torch.bfloat16))
+
+
+def test_broadcast_views_are_accepted():
+    """Losses that hand backward an expanded gradient (stride 0 along a summed axis) and keys
+    expanded over heads (stride 0 on H) run, as the reference's stride-generic launch lets them
+    (simplicial/triton_impl.py:38-45), and give what the materialised tensors give."""
+    import simplical_attn_amd as sa
+    dev = torch.device("cuda:0")
+    inp = make_inputs(2, 70, 3, 64, seed=21, dtype=torch.float32)
+    attn = sa.TwoSimplicialAttention(64, 12, 5)
+
+    def grads_of(loss_of, k1_of=lambda t: t):
+        leaves = [x.to(dev).requires_grad_(True) for x in inp[:5]]
+        args = list(leaves)
+        args[1] = k1_of(leaves[1])
+        loss_of(attn(*args)).backward()
+        return [t.grad for t in leaves]
+
+    w = inp[5].to(dev)
+    # sum over N: autograd expands a [B,H,D] gradient with stride 0 on N
+    a = grads_of(lambda o: (o.sum(dim=1) * w[:, 0]).sum())
+    b = grads_of(lambda o: (o * w[:, :1].expand_as(o).contiguous()).sum())
+    for x, y in zip(a, b):
+        assert torch.allclose(x, y, rtol=1e-5, atol=1e-6)
+    # sum over everything but D: strides (0, 0, 0, 1)
+    a = grads_of(lambda o: (o.sum(dim=(0, 1, 2)) * w[0, 0, 0]).sum())
+    b = grads_of(lambda o: (o * w[:1, :1, :1].expand_as(o).contiguous()).sum())
+    for x, y in zip(a, b):
+        assert torch.allclose(x, y, rtol=1e-5, atol=1e-6)
+    # one key head shared by all query heads (MQA): k1 expanded over H
+    a = grads_of(lambda o: (o * w).sum(), k1_of=lambda t: t[:, :, :1].expand(-1, -1, 3, -1))
+    b = grads_of(lambda o: (o * w).sum(), k1_of=lambda t: t[:, :, :1].expand(-1, -1, 3, -1).contiguous())
+    for x, y in zip(a, b):
+        assert torch.allclose(x, y, rtol=1e-5, atol=1e-6)
+    want = oracle_all([inp[0], inp[1][:, :, :1].expand(-1, -1, 3, -1), *inp[2:]], 12, 5)
+    out = attn(inp[0].to(dev), inp[1].to(dev)[:, :, :1].expand(-1, -1, 3, -1), *[x.to(dev) for x in inp[2:5]])
+    assert torch.allclose(out.cpu().double(), want["out"], rtol=1e-5, atol=1e-5)
