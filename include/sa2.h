@@ -40,7 +40,9 @@ typedef enum sa2_status {
     SA2_ERR_WORKSPACE_TOO_SMALL = -6,
     SA2_ERR_LAUNCH_FAILED = -7,  /* hipGetLastError() after a launch */
     SA2_ERR_UNSUPPORTED = -8,    /* a forced kernel path does not support the shape/dtype */
-    SA2_ERR_TOO_LARGE = -9       /* an index would overflow the kernels' 32-bit grid */
+    SA2_ERR_TOO_LARGE = -9,      /* an index would overflow the kernels' 32-bit grid */
+    SA2_ERR_STATIC_WORKSPACE = -10 /* sa2_backward_static_workspace: the problem needs more than
+                                      SA2_STATIC_WORKSPACE_BYTES, or the array's address is unavailable */
 } sa2_status;
 
 typedef enum sa2_dtype { SA2_F32 = 0, SA2_BF16 = 1, SA2_F16 = 2 } sa2_dtype;
@@ -63,8 +65,10 @@ int sa2_version(void);
 /* Static, NUL-terminated description of a status code. */
 const char* sa2_strerror(int status);
 
-/* 1 if sa2_forward / sa2_backward would take the MFMA kernels for this
- * problem under SA2_FLAG_AUTO, 0 if they would take the generic kernels. */
+/* 1 if sa2_forward would take the MFMA kernels for this problem under SA2_FLAG_AUTO
+ * (given 16-byte aligned rows), 0 if it would take the generic kernels.  It answers for
+ * the forward only: sa2_backward additionally falls back to the generic kernels for
+ * fp16 or D = 32 problems whose K' window exceeds what its on-chip kernels hold. */
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype);
 
 /*
@@ -113,6 +117,27 @@ int sa2_backward(const void* q, const void* k1, const void* k2, const void* v1, 
                  const int64_t* strides,
                  int w1, int w2, float scale, float k2_bias, float v2_bias,
                  int dtype, int window_inclusive, unsigned flags, void* hip_stream);
+
+/*
+ * sa2_backward for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart
+ * in the reference.  Same arguments, kernels and results as sa2_backward, minus the
+ * workspace: that is a file-scope device array of SA2_STATIC_WORKSPACE_BYTES inside the
+ * library, one copy per GPU, held until the process ends.  The call itself allocates and
+ * frees nothing.  A problem with sa2_bwd_workspace_bytes(...) > SA2_STATIC_WORKSPACE_BYTES
+ * returns SA2_ERR_STATIC_WORKSPACE and launches nothing.  All calls on one GPU share the
+ * array (the kernels overwrite what they read from it, so nothing needs clearing between
+ * calls): calls that overlap on one GPU - different streams, or host threads - race;
+ * calls on one stream are safe.
+ */
+#define SA2_STATIC_WORKSPACE_BYTES (64u << 20)
+int sa2_backward_static_workspace(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                                  const void* out, const void* dout, const float* lse,
+                                  void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
+                                  int B, int N, int H, int D,
+                                  const int64_t* strides,
+                                  int w1, int w2, float scale, float k2_bias, float v2_bias,
+                                  int dtype, int window_inclusive, unsigned flags, void* hip_stream);
 
 /*
  * Row term of the softmax Jacobian, dsum[b,h,i] = sum_d dout[b,i,h,d]*out[b,i,h,d]

@@ -8,8 +8,9 @@ LIB_PATH = os.environ.get("SA2_LIBRARY", os.path.join(_PKG, "lib", "libsa2_hip.s
 # Symbols include/sa2.h declares; the ABI test checks that all of them resolve.
 EXPORTED_SYMBOLS = (
     "sa2_version", "sa2_strerror", "sa2_uses_mfma", "sa2_forward",
-    "sa2_bwd_workspace_bytes", "sa2_backward", "sa2_rowdot",
+    "sa2_bwd_workspace_bytes", "sa2_backward", "sa2_backward_static_workspace", "sa2_rowdot",
 )
+STATIC_WORKSPACE_BYTES = 64 << 20
 
 SA2_F32, SA2_BF16, SA2_F16 = 0, 1, 2
 FLAG_AUTO, FLAG_FORCE_GENERIC, FLAG_FORCE_MFMA = 0, 1, 2
@@ -52,6 +53,10 @@ def load():
     lib.sa2_backward.restype = c_int
     lib.sa2_backward.argtypes = ([c_void_p] * 13 + [c_void_p, c_size_t] + [c_int] * 4 + [i64p]
                                  + [c_int, c_int, c_float, c_float, c_float] + [c_int, c_int, c_uint, c_void_p])
+    lib.sa2_backward_static_workspace.restype = c_int
+    lib.sa2_backward_static_workspace.argtypes = ([c_void_p] * 13 + [c_int] * 4 + [i64p]
+                                                  + [c_int, c_int, c_float, c_float, c_float]
+                                                  + [c_int, c_int, c_uint, c_void_p])
     lib.sa2_rowdot.restype = c_int
     lib.sa2_rowdot.argtypes = [c_void_p] * 3 + [c_int] * 4 + [i64p, c_int, c_void_p]
     _lib = lib

@@ -1,6 +1,7 @@
 // extern "C" boundary: argument validation and kernel-path selection.
 // No allocation and no synchronisation.  The only process state is set-up that happens once and
-// never depends on a call's arguments: each kernel's LDS limit (allow_full_lds).
+// never depends on a call's arguments: each kernel's LDS limit (allow_full_lds) and, for
+// sa2_backward_static_workspace, the per-device address of the library's own workspace array.
 #include <string.h>
 
 #include <mutex>
@@ -31,6 +32,11 @@ bool allow_full_lds(const void* kernel) {
 }
 
 }  // namespace sa2
+
+// Workspace of sa2_backward_static_workspace: one copy per GPU the library runs on, held until
+// the process ends.  In host code this name is only a handle for hipGetSymbolAddress; the
+// device address it yields (per device) is what the kernels are given.
+static __device__ __align__(256) unsigned char scratch[SA2_STATIC_WORKSPACE_BYTES];
 
 namespace {
 
@@ -71,6 +77,25 @@ bool strides_ok(const int64_t* strides, int count, int B, int N, int H) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Device address of `scratch` on the current device, looked up on the first call on that
+// device (with that device current) and kept; NULL if the lookup fails.
+void* static_workspace() {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static void* address[MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!address[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        address[dev] = ptr;
+    }
+    return address[dev];
+}
+
+size_t dsum_bytes(int B, int N, int H) { return align_up((size_t)B * H * N * sizeof(float), 256); }
+
 bool pick_mfma(const Problem& p, int dtype, unsigned flags, bool backward, int* status) {
     *status = SA2_OK;
     if (flags & SA2_FLAG_FORCE_GENERIC) return false;
@@ -99,6 +124,8 @@ const char* sa2_strerror(int status) {
         case SA2_ERR_LAUNCH_FAILED: return "a HIP kernel launch failed";
         case SA2_ERR_UNSUPPORTED: return "the forced kernel path does not support this shape, dtype or layout";
         case SA2_ERR_TOO_LARGE: return "problem too large for the kernels' 32-bit grid (B*H*N must be < 2^31)";
+        case SA2_ERR_STATIC_WORKSPACE: return "the problem needs more workspace than the library's own SA2_STATIC_WORKSPACE_BYTES, or "
+                                              "the address of that array could not be obtained on this device";
     }
     return "unknown sa2 status";
 }
@@ -195,6 +222,23 @@ int sa2_backward(const void* q, const void* k1, const void* k2, const void* v1, 
     const bool mfma = pick_mfma(p, dtype, flags, true, &rc);
     if (rc != SA2_OK) return rc;
     return mfma ? launch_mfma_bwd(p, dtype, st) : launch_generic_bwd(p, dtype, st);
+}
+
+int sa2_backward_static_workspace(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                                  const void* out, const void* dout, const float* lse,
+                                  void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
+                                  int B, int N, int H, int D, const int64_t* strides,
+                                  int w1, int w2, float scale, float k2_bias, float v2_bias,
+                                  int dtype, int window_inclusive, unsigned flags, void* hip_stream) {
+    int rc = check_dims(B, N, H, D, w1, w2, dtype, window_inclusive);
+    if (rc != SA2_OK) return rc;
+    const size_t need = sa2_bwd_workspace_bytes(B, N, H, D, window_inclusive ? w1 : w1 - 1,
+                                                window_inclusive ? w2 : w2 - 1, dtype, flags);
+    if (need == 0 || need > (size_t)SA2_STATIC_WORKSPACE_BYTES) return SA2_ERR_STATIC_WORKSPACE;
+    void* ws = static_workspace();
+    if (!ws) return SA2_ERR_STATIC_WORKSPACE;
+    return sa2_backward(q, k1, k2, v1, v2, out, dout, lse, dq, dk1, dk2, dv1, dv2, ws, SA2_STATIC_WORKSPACE_BYTES,
+                        B, N, H, D, strides, w1, w2, scale, k2_bias, v2_bias, dtype, window_inclusive, flags, hip_stream);
 }
 
 int sa2_rowdot(const void* out, const void* dout, float* dsum, int B, int N, int H, int D,

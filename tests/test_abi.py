@@ -35,7 +35,7 @@ def test_version_and_strerror(lib):
     assert lib.sa2_version() == 1
     assert lib.sa2_strerror(0) == b"success"
     seen = set()
-    for code in range(-9, 0):
+    for code in range(-10, 0):
         msg = lib.sa2_strerror(code)
         assert msg and msg not in seen
         seen.add(msg)
