@@ -20,6 +20,10 @@ PyTorch "gold standard":
                                                (simplicial/reference.py:68-74)
     scale        defaults to 1/sqrt(D)         (simplicial/reference.py:29-30)
 
+The reference's device kernels mask half-open windows instead, (i-w, i], w keys
+(simplicial/kernels.py:133-136: ``q_idx - w < kv_idx``).  ``inclusive=False`` selects that
+convention in every function below; the default is reference.py's.
+
 The reference never returns a log-sum-exp; the only definition in the
 reference is the device kernels' ``m + log(l)`` (simplicial/kernels.py:164).
 Here LSE is defined so that ``exp(s - LSE)`` is exactly the oracle's normalised
@@ -32,6 +36,9 @@ How each function is pinned (tests/test_oracle.py):
                       (pins the w+1-key window convention), row-0 closed form,
                       swap symmetry, bias == shifted input.
   forward_windowed    the same checks, plus equality with literal_loop.
+  inclusive=False     the same brute force with strict lower bounds (j > i-w1, k > i-w2), the
+                      q = 0 closed form with min(i+1, w) keys per window, and the published
+                      triple counts of the half-open convention.
   grads_windowed      torch.autograd.gradcheck (fp64) on forward_windowed, the
                       closed-form gradients of the dense brute force (autograd
                       through an independent einsum formulation), and central
@@ -48,7 +55,7 @@ def default_scale(head_dim):
     return 1.0 / math.sqrt(head_dim)
 
 
-def literal_loop(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0):
+def literal_loop(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0, inclusive=True):
     """Literal-order restatement: queries, then K keys, then K' keys, one
     weight at a time, numerator accumulated in the input dtype and the
     denominator in fp32 (simplicial/reference.py:39-74; the fp32 denominator is
@@ -56,13 +63,17 @@ def literal_loop(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0
     fp64 here, so that an fp64 run is a truth source.  Vectorised over
     (batch, head) only.  Feasible for small shapes (N*(w1+1)*(w2+1) steps)."""
     B, N, H, D = q.shape
+    _check_windows(w1, w2, inclusive)
     if scale is None:
         scale = default_scale(D)
     k2b = k2 + k2_bias
     v2b = v2 + v2_bias
     out = torch.zeros_like(q)
     for i in range(N):
-        j_lo, k_lo = max(0, i - w1), max(0, i - w2)
+        if inclusive:
+            j_lo, k_lo = max(0, i - w1), max(0, i - w2)              # reference.py:41-45
+        else:
+            j_lo, k_lo = max(0, i - w1 + 1), max(0, i - w2 + 1)      # kernels.py:133-136
         qi = q[:, i]                                   # [B,H,D]
         num = torch.zeros_like(qi)
         den = torch.zeros(B, H, 1, dtype=torch.float32 if q.dtype != torch.float64 else torch.float64)
@@ -77,15 +88,21 @@ def literal_loop(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0
     return out
 
 
-def _band(rows, cols, w):
-    """mask[r,c] = (rows[r]-w <= cols[c] <= rows[r])."""
+def _check_windows(w1, w2, inclusive):
+    if w1 < 0 or w2 < 0 or (not inclusive and (w1 < 1 or w2 < 1)):
+        raise ValueError("windows must be >= 0 (>= 1 for the half-open convention, which would hold no key)")
+
+
+def _band(rows, cols, w, inclusive=True):
+    """mask[r,c] = (rows[r]-w <= cols[c] <= rows[r]); with inclusive=False the lower
+    bound is strict (simplicial/kernels.py:133-136)."""
     r = rows[:, None]
     c = cols[None, :]
-    return (c <= r) & (c >= r - w)
+    return (c <= r) & ((c >= r - w) if inclusive else (c > r - w))
 
 
 def forward_windowed(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0,
-                     rows=None, chunk=32, compute_dtype=None):
+                     rows=None, chunk=32, compute_dtype=None, inclusive=True):
     """Vectorised restatement of the same arithmetic on a range of query rows.
 
     rows = (r0, r1) restricts the computation to queries r0 <= i < r1 (outputs
@@ -99,6 +116,7 @@ def forward_windowed(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias
     O = sum w v / (sum w + 1e-8) holds for logits of any magnitude.
     """
     B, N, H, D = q.shape
+    _check_windows(w1, w2, inclusive)
     if scale is None:
         scale = default_scale(D)
     if compute_dtype is None:
@@ -117,7 +135,7 @@ def forward_windowed(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias
         kk = torch.arange(k0, c1)
         qk = qf[:, :, c0:c1, None, :] * k2f[:, :, None, k0:c1, :]        # [B,H,i,k,D]
         s = torch.matmul(qk, k1f[:, :, None, j0:c1, :].transpose(-1, -2)) * scale   # [B,H,i,k,j]
-        mask = _band(ii, kk, w2)[:, :, None] & _band(ii, jj, w1)[:, None, :]      # [i,k,j]
+        mask = _band(ii, kk, w2, inclusive)[:, :, None] & _band(ii, jj, w1, inclusive)[:, None, :]      # [i,k,j]
         s = s.masked_fill(~mask, float("-inf"))
         m = s.amax(dim=(-1, -2), keepdim=True)                           # [B,H,i,1,1]
         w = torch.exp(s - m)
@@ -137,7 +155,7 @@ def forward_windowed(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias
 
 
 def grads_windowed(q, k1, k2, v1, v2, dout, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0,
-                   rows=None, chunk=32, compute_dtype=None):
+                   rows=None, chunk=32, compute_dtype=None, inclusive=True):
     """Gradients of sum(O*dout) over the query rows in ``rows`` with respect to
     the five inputs, by autograd through forward_windowed, one chunk at a
     time.  ``dout`` has the same row range as the output.  Returns
@@ -152,7 +170,7 @@ def grads_windowed(q, k1, k2, v1, v2, dout, w1, w2, scale=None, k2_bias=0.0, v2_
     for c0 in range(r0, r1, chunk):
         c1 = min(r1, c0 + chunk)
         o, lse = forward_windowed(*leaves, w1, w2, scale, k2_bias, v2_bias,
-                                  rows=(c0, c1), chunk=chunk, compute_dtype=compute_dtype)
+                                  rows=(c0, c1), chunk=chunk, compute_dtype=compute_dtype, inclusive=inclusive)
         (o * dout[:, c0 - r0:c1 - r0].to(compute_dtype)).sum().backward()
         outs.append(o.detach())
         lses.append(lse.detach())
@@ -160,10 +178,11 @@ def grads_windowed(q, k1, k2, v1, v2, dout, w1, w2, scale=None, k2_bias=0.0, v2_
     return (torch.cat(outs, dim=1), torch.cat(lses, dim=2), *grads)
 
 
-def count_triples(B, N, H, w1, w2):
+def count_triples(B, N, H, w1, w2, inclusive=True):
     """Number of valid (i,j,k) triples summed over batch and heads:
-    B*H*sum_i (min(i,w1)+1)*(min(i,w2)+1) (windows of simplicial/reference.py:41-45)."""
+    B*H*sum_i (min(i,w1)+1)*(min(i,w2)+1) (windows of simplicial/reference.py:41-45), or
+    B*H*sum_i min(i+1,w1)*min(i+1,w2) for the half-open windows of simplicial/kernels.py:133-136."""
     t = 0
     for i in range(N):
-        t += (min(i, w1) + 1) * (min(i, w2) + 1)
+        t += (min(i, w1) + 1) * (min(i, w2) + 1) if inclusive else min(i + 1, w1) * min(i + 1, w2)
     return B * H * t

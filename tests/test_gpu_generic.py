@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import simplicial_oracle as orc
-from tests.util import assert_close_rel, make_inputs, oracle_all, rel_err, run_device
+from tests.util import assert_close_rel, make_inputs, oracle_all, record, rel_err, run_device
 
 pytestmark = pytest.mark.gpu
 GENERIC = 1
@@ -24,6 +24,8 @@ def test_config1_fp32_forward_matches_literal_oracle():
     o64, lse64 = orc.forward_windowed(*[x.double() for x in inp[:5]], 32, 16)
     assert torch.allclose(got["out"].cpu().double(), o64, rtol=1e-5, atol=1e-5)
     assert torch.allclose(got["lse"].cpu().double(), lse64, rtol=1e-5, atol=1e-5)
+    record("c1 fp32 B1 H2 N128 D64 w32/16", "out", got["out"], o64)
+    record("c1 fp32 B1 H2 N128 D64 w32/16", "lse", got["lse"], lse64)
 
 
 def test_config1_fp32_gradients():
@@ -32,6 +34,7 @@ def test_config1_fp32_gradients():
     want = oracle_all(inp, 32, 16)
     for name in ("dq", "dk1", "dk2", "dv1", "dv2"):
         assert torch.allclose(got[name].cpu().double(), want[name], rtol=1e-5, atol=1e-5), name
+        record("c1 fp32 B1 H2 N128 D64 w32/16", name, got[name], want[name])
 
 
 @pytest.mark.parametrize("shape", [(1, 32, 1, 16), (2, 64, 2, 32), (4, 128, 4, 64), (1, 256, 8, 128), (1, 40, 2, 256),
@@ -174,6 +177,12 @@ def test_half_open_window_convention():
     a, la = sa.simplicial_forward(*inp, 6, 4, flags=GENERIC, window_inclusive=False)
     b, lb = sa.simplicial_forward(*inp, 5, 3, flags=GENERIC, window_inclusive=True)
     assert torch.equal(a, b) and torch.equal(la, lb)
+    # and against the oracle's own half-open windows, forward and gradients, to the fp32 bar
+    host = make_inputs(1, 40, 2, 16, seed=13)
+    got = run_device(host, 6, 4, flags=GENERIC, inclusive=False)
+    want = oracle_all(host, 6, 4, inclusive=False)
+    for name in ("out", "lse", "dq", "dk1", "dk2", "dv1", "dv2"):
+        assert torch.allclose(got[name].cpu().double(), want[name], rtol=1e-5, atol=1e-5), name
 
 
 def test_error_codes():

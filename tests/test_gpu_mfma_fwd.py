@@ -24,6 +24,12 @@ def fwd(inp, w1, w2, scale=None, kb=0.0, vb=0.0, flags=MFMA):
     return sa.simplicial_forward(*[x.to(dev) for x in inp[:5]], w1, w2, scale, kb, vb, flags=flags)
 
 
+def sa_forward_half_open(inp, w1, w2):
+    import simplical_attn_amd as sa
+    dev = torch.device("cuda:0")
+    return sa.simplicial_forward(*[x.to(dev) for x in inp[:5]], w1, w2, flags=MFMA, window_inclusive=False)
+
+
 def oracle_rows(inp, w1, w2, rows, scale=None, kb=0.0, vb=0.0, dtype=torch.float64):
     return orc.forward_windowed(*[x.to(dtype) for x in inp[:5]], w1, w2, scale, kb, vb, rows=rows,
                                 compute_dtype=dtype)
@@ -50,8 +56,8 @@ def test_small_shapes_vs_oracle(case):
     inp = make_inputs(B, N, H, D, seed=N + D + w1, dtype=torch.bfloat16, with_dout=False)
     out, lse = fwd(inp, w1, w2, None, kb, vb)
     want, want_lse = oracle_rows(inp, w1, w2, None, None, kb, vb)
-    assert_close_rel(out, want, BF16_TOL, "out")
-    assert_close_rel(lse, want_lse, BF16_TOL, "lse")
+    assert_close_rel(out, want, BF16_TOL, "out", label="small shapes bf16 (fwd)")
+    assert_close_rel(lse, want_lse, BF16_TOL, "lse", label="small shapes bf16 (fwd)")
 
 
 FP16_CASES = [SMALL[1], SMALL[4], SMALL[6], SMALL[7]]
@@ -109,8 +115,8 @@ def test_config2_forward():
     out, lse = fwd(inp, 512, 32)
     for rows in ((0, 96), (480, 576), (1990, 2048)):
         want, want_lse = oracle_rows(inp, 512, 32, rows, dtype=torch.float32)
-        assert_close_rel(out[:, rows[0]:rows[1]], want, BF16_TOL, "out rows %s" % (rows,))
-        assert_close_rel(lse[:, :, rows[0]:rows[1]], want_lse, BF16_TOL, "lse rows %s" % (rows,))
+        assert_close_rel(out[:, rows[0]:rows[1]], want, BF16_TOL, "out rows %s" % (rows,), label="c2 bf16 B2 H8 N2048 D64 w512/32")
+        assert_close_rel(lse[:, :, rows[0]:rows[1]], want_lse, BF16_TOL, "lse rows %s" % (rows,), label="c2 bf16 B2 H8 N2048 D64 w512/32")
     ref, ref_lse = fwd(inp, 512, 32, flags=GENERIC)
     assert_close_rel(out, ref.float().cpu(), BF16_TOL, "out vs generic kernel")
     assert_close_rel(lse, ref_lse.cpu(), BF16_TOL, "lse vs generic kernel")
@@ -125,6 +131,14 @@ def test_config4_forward_headline_shape():
         want, want_lse = oracle_rows(inp, 512, 32, rows, dtype=torch.float32)
         assert_close_rel(out[:, rows[0]:rows[1]], want, BF16_TOL, "out rows %s" % (rows,))
         assert_close_rel(lse[:, :, rows[0]:rows[1]], want_lse, BF16_TOL, "lse rows %s" % (rows,))
+    # the half-open windows of the reference's device kernels at the same shape (w 512/32 then
+    # reach 511/31: no pre-pass, a partial last round), oracle with its own half-open masks
+    out_h, lse_h = sa_forward_half_open(inp, 512, 32)
+    for rows in ((0, 40), (500, 540), (8160, 8192)):
+        want, want_lse = orc.forward_windowed(*[x.float() for x in inp[:5]], 512, 32, rows=rows,
+                                              compute_dtype=torch.float32, inclusive=False)
+        assert_close_rel(out_h[:, rows[0]:rows[1]], want, BF16_TOL, "half-open out rows %s" % (rows,))
+        assert_close_rel(lse_h[:, :, rows[0]:rows[1]], want_lse, BF16_TOL, "half-open lse rows %s" % (rows,))
     ref, ref_lse = fwd(inp, 512, 32, flags=GENERIC)
     assert_close_rel(out, ref.float().cpu(), BF16_TOL, "out vs generic kernel")
     assert_close_rel(lse, ref_lse.cpu(), BF16_TOL, "lse vs generic kernel")

@@ -232,3 +232,72 @@ def test_count_triples():
             for k in range(max(0, i - 2), i + 1):
                 n += 1
     assert orc.count_triples(2, 20, 3, 5, 2) == 6 * n
+
+
+# ---- the half-open windows of the reference's device kernels (simplicial/kernels.py:133-136) ----
+
+def brute_force_half_open(q, k1, k2, v1, v2, w1, w2, scale, k2_bias=0.0, v2_bias=0.0):
+    """brute_force with the masks as the device kernels write them:
+    q_idx - w < kv_idx <= q_idx on both sides."""
+    B, N, H, D = q.shape
+    s = torch.einsum("bihd,bjhd,bkhd->bhijk", q, k1, k2 + k2_bias) * scale
+    idx = torch.arange(N)
+    i, j, k = idx[:, None, None], idx[None, :, None], idx[None, None, :]
+    mask = ((i - w1) < j) & (j <= i) & ((i - w2) < k) & (k <= i)
+    w = torch.exp(s) * mask
+    tot = w.sum(dim=(-1, -2))
+    out = torch.einsum("bhijk,bjhd,bkhd->bihd", w, v1, v2 + v2_bias) / (tot.permute(0, 2, 1)[..., None] + 1e-8)
+    return out, torch.log(tot + 1e-8)
+
+
+@pytest.mark.parametrize("case", [
+    (1, 12, 1, 4, 3, 2, 0.0, 0.0),
+    (2, 20, 2, 8, 5, 7, 0.1, -0.2),
+    (1, 24, 2, 6, 30, 4, 1.0, 0.5),      # w1 >= N
+    (1, 16, 1, 8, 1, 1, 0.0, 0.0),       # single (i,i,i) triple
+    (1, 33, 3, 5, 2, 9, -0.1, 0.2),
+])
+def test_half_open_windows_match_brute_force(case):
+    B, N, H, D, w1, w2, kb, vb = case
+    t = five(B, N, H, D, seed=N + 100)
+    dout = rnd((B, N, H, D), 77)
+    scale = 0.41
+    leaves = [x.clone().requires_grad_(True) for x in t]
+    ref, ref_lse = brute_force_half_open(*leaves, w1, w2, scale, kb, vb)
+    (ref * dout).sum().backward()
+    lit = orc.literal_loop(*t, w1, w2, scale, kb, vb, inclusive=False)
+    res = orc.grads_windowed(*t, dout, w1, w2, scale, kb, vb, chunk=7, inclusive=False)
+    assert torch.allclose(lit, ref.detach(), rtol=1e-11, atol=1e-12)
+    assert torch.allclose(res[0], ref.detach(), rtol=1e-11, atol=1e-12)
+    assert torch.allclose(res[1], ref_lse.detach(), rtol=1e-11, atol=1e-12)
+    for g, leaf in zip(res[2:], leaves):
+        assert torch.allclose(g, leaf.grad, rtol=1e-9, atol=1e-11)
+    # and it differs from the closed windows of the same w (one key more per side)
+    closed, _ = orc.forward_windowed(*t, w1, w2, scale, kb, vb)
+    assert not torch.allclose(closed[:, 1:], ref.detach()[:, 1:], rtol=1e-3, atol=1e-3)
+
+
+def test_half_open_zero_query_counts_w_keys():
+    """q = 0: LSE_i = log(|J(i)|*|K(i)| + 1e-8) with |J(i)| = min(i+1, w1): w keys, not w+1."""
+    B, N, H, D, w1, w2 = 1, 25, 1, 4, 6, 3
+    _, k1, k2, v1, v2 = five(B, N, H, D, seed=8)
+    q = torch.zeros_like(k1)
+    out, lse = orc.forward_windowed(q, k1, k2, v1, v2, w1, w2, 1.0, 0.0, 0.25, inclusive=False)
+    for i in range(N):
+        nj, nk = min(i + 1, w1), min(i + 1, w2)
+        want = v1[:, i - nj + 1:i + 1].sum(1) * (v2[:, i - nk + 1:i + 1] + 0.25).sum(1) / (nj * nk + 1e-8)
+        assert torch.allclose(out[:, i], want, rtol=1e-12, atol=1e-13)
+        assert abs(lse[0, 0, i].item() - math.log(nj * nk + 1e-8)) < 1e-12
+
+
+def test_half_open_rejects_empty_windows_and_counts_triples():
+    t = five(1, 6, 1, 4, seed=2)
+    with pytest.raises(ValueError):
+        orc.forward_windowed(*t, 0, 3, inclusive=False)
+    with pytest.raises(ValueError):
+        orc.literal_loop(*t, 3, 0, inclusive=False)
+    assert orc.count_triples(1, 128, 2, 32, 16, inclusive=False) == 113840
+    assert orc.count_triples(1, 8192, 16, 512, 32, inclusive=False) == 2080418560
+    n = sum(1 for i in range(20) for j in range(20) for k in range(20)
+            if i - 5 < j <= i and i - 2 < k <= i)
+    assert orc.count_triples(2, 20, 3, 5, 2, inclusive=False) == 6 * n
