@@ -11,17 +11,27 @@ w1=512 w2=32.  Prints ONE JSON line:
   metric/value   forward+backward algorithmic TFLOP/s: 16*D*T flops per step,
                  T = number of valid (i,j,k) triples (matmul flops only, 2 per
                  MAC: 4*D*T forward, 12*D*T backward)
-  roofline       the kernel that dominates the step, against the bf16 dense MFMA
-                 peak (achieved = that kernel's algorithmic flops / its duration,
-                 measured here with events on the launch stream)
+  roofline       the single kernel that dominates the step, against the bf16 dense
+                 MFMA peak (achieved = that kernel's algorithmic flops / its duration,
+                 measured here with events on the launch stream); `mfma_busy` and
+                 `traffic` are rocprofv3 counter results read from profiles/
+                 (measured in separate profiler runs of this same script)
   kernels        the same for every kernel group of the step, plus HBM GB/s
+  clock          shader clock observed while the kernels run (a spin kernel on a
+                 second stream counts device cycles between two events) and the
+                 peak recomputed from it: CUs x 4096 flop/clk x clock
   cpu_baseline   the CPU oracle (a port of the reference's PyTorch loop) timed on
                  this host on a bounded sample of the same workload
+  cpu_reference_literal   the literal triple loop of the reference (reference.py:39-74,
+                 restated in oracle/) timed at configuration c1, with its cost per
+                 loop iteration and the extrapolation to this workload
 """
 import argparse
+import glob
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -30,9 +40,10 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK_BF16_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
+PEAK_BF16_TFLOPS = 2516.6     # published: 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
 PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+BF16_FLOP_PER_CLK_PER_CU = 4096
 
 WORKLOADS = {
     # name: (B, N, H, D, w1, w2, seed, qk_std)
@@ -41,13 +52,22 @@ WORKLOADS = {
     "c5": (1, 32768, 8, 128, 1024, 64, 4, 0.5),
 }
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
-# scaled by the same counters on a plain copy kernel; None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 864.2e6,                # pre-pass 419.7 MB + fast kernel 443.4 MB + repair launch 1.1 MB
-    ("c4", "backward_k_side"): 632.2e6,        # mfma_bwd_kv_kernel
-    ("c4", "backward_kprime_side"): 1954.0e6,  # pre-pass 766.5 MB + mfma_bwd_kp_kernel 886.0 MB + dq_sum 301.5 MB
-}
+
+
+def profile_keys():
+    """Counter results of the tracked rocprofv3 summaries: every line of profiles/*.md of the form
+    `<workload>.<kernel group>.<quantity> = <number>` (HBM bytes per launch from FETCH_SIZE and
+    WRITE_SIZE scaled by a copy kernel; matrix-pipe busy fraction from SQ_VALU_MFMA_BUSY_CYCLES).
+    They are measured under the profiler, not in this run: a key that is missing reads as None."""
+    keys, sources = {}, {}
+    pat = re.compile(r"^([a-z0-9]+)\.([a-z_]+)\.([a-z_]+) = ([-+0-9.eE]+)\s*$")
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        for line in open(path):
+            m = pat.match(line.strip())
+            if m:
+                keys[(m.group(1), m.group(2), m.group(3))] = float(m.group(4))
+                sources[m.group(1)] = os.path.relpath(path, ROOT)
+    return keys, sources
 
 
 def count_triples(B, N, H, w1, w2):
@@ -77,6 +97,51 @@ def time_gpu(fn, steps, warmup):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / steps
+
+
+def observed_clock_mhz(fn, ms_per_call, spin_ms=60.0):
+    """Shader clock while `fn` keeps the GPU busy: a one-thread spin kernel on a second stream
+    waits for a given number of ticks of the device's cycle counter between two events, and
+    calls of `fn` queued right behind it on the launch stream run for its whole duration.  The
+    spin is launched on an idle (but just warmed) GPU so that it starts at once and the events
+    bracket exactly its ticks.  (The spinning wavefront takes one CU's slot for its duration;
+    this is a measurement of its own, outside the timed region.)"""
+    side = torch.cuda.Stream()
+    cycles = int(2.4e6 * spin_ms)                      # lasts about `spin_ms` at 2.4 GHz
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        e0.record()
+        torch.cuda._sleep(cycles)
+        e1.record()
+    for _ in range(int(math.ceil(1.4 * spin_ms / ms_per_call)) + 2):
+        fn()
+    torch.cuda.synchronize()
+    return cycles / e0.elapsed_time(e1) / 1e3
+
+
+def cpu_reference_literal(target_iterations, target_name):
+    """The reference's literal triple loop (queries x K keys x K' keys, one weight at a time;
+    simplicial/reference.py:39-74 as restated in oracle/) at configuration c1, the only one it
+    finishes in seconds, and its per-iteration cost extrapolated by iteration count."""
+    from oracle import simplicial_oracle as orc
+    B, N, H, D, w1, w2 = 1, 128, 2, 64, 32, 16
+    g = torch.Generator().manual_seed(0)
+    tens = [torch.randn(B, N, H, D, generator=g, dtype=torch.float32) for _ in range(5)]
+    iterations = sum((min(i, w1) + 1) * (min(i, w2) + 1) for i in range(N))     # (B, H) is vectorised
+    t0 = time.perf_counter()
+    orc.literal_loop(*tens, w1, w2)
+    dt = time.perf_counter() - t0
+    return {
+        "workload": "c1: fp32 forward B=1 H=2 N=128 D=64 w1=32 w2=16", "kind": "port", "ms": dt * 1e3,
+        "iterations": iterations, "us_per_iteration": dt / iterations * 1e6, "cores": torch.get_num_threads(),
+        "extrapolated": {"workload": target_name, "iterations": target_iterations,
+                         "hours_forward": dt / iterations * target_iterations / 3600.0,
+                         "note": "per-iteration cost at c1 x iteration count; an extrapolation, not a measurement "
+                                 "(the loop's tensors grow with B*H*D, so this is a lower bound)"},
+    }
 
 
 def cpu_baseline(name, cfg, budget_rows):
@@ -181,7 +246,7 @@ def main():
     out, lse = sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2)
     ksteps = max(5, args.steps)
     fwd_ms = time_gpu(lambda: sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2), ksteps, 2)
-    rowdot_ms = time_gpu(lambda: sa.compute_D_kernel(dout, out), ksteps, 2)
+    rowdot_ms = time_gpu(lambda: sa.simplicial_rowdot(dout, out), ksteps, 2)
     bwd_all_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2), ksteps, 2)
     bwd_k1_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2,
                                                         needs=(False, True, False, True, False)), ksteps, 2) - rowdot_ms
@@ -192,35 +257,66 @@ def main():
     # two MFMA kernels (each owns two output contractions, 4*D*T, and half of the S / dP
     # recomputation that the pair shares, 2*D*T).
     half_bwd = bwd_flops / 2
+    keys, key_sources = profile_keys()
+    wl = args.workload
     kernels = {
         "forward": {"kernel": "mfma_fwd_kernel<%d> (pre-pass + fast kernel + repair launch)" % D, "ms": fwd_ms,
-                    "flops": fwd_flops},
-        "backward_k_side": {"kernel": "mfma_bwd_kv_kernel<%d> (dK, dV)" % D, "ms": bwd_k1_ms, "flops": half_bwd},
+                    "flops": fwd_flops, "launches": 3},
+        "backward_k_side": {"kernel": "mfma_bwd_kv_kernel<%d> (dK, dV)" % D, "ms": bwd_k1_ms, "flops": half_bwd,
+                            "launches": 1},
         "backward_kprime_side": {"kernel": "mfma_bwd_kp_kernel<%d> (pre-pass + main) + dq_sum (dQ, dK', dV')" % D, "ms": bwd_rest_ms,
-                                 "flops": half_bwd},
+                                 "flops": half_bwd, "launches": 3},
     }
-    for k in kernels.values():
+    for name, k in kernels.items():
         k["tflops"] = k["flops"] / k["ms"] / 1e9
         k["frac_bf16_peak"] = k["tflops"] / PEAK_BF16_TFLOPS
+        k["mfma_busy"] = keys.get((wl, name, "mfma_busy"))          # rocprofv3, from profiles/
+        k["traffic"] = keys.get((wl, name, "traffic_bytes"))
     kernels["forward"]["hbm_gbs"] = fwd_bytes / fwd_ms / 1e6
     kernels["backward"] = {"ms": bwd_all_ms, "tflops": bwd_flops / bwd_all_ms / 1e9, "hbm_gbs": bwd_bytes / bwd_all_ms / 1e6,
                            "frac_bf16_peak": bwd_flops / bwd_all_ms / 1e9 / PEAK_BF16_TFLOPS}
     kernels["rowdot"] = {"ms": rowdot_ms, "hbm_gbs": (4 * E + 4 * B * H * N) / rowdot_ms / 1e6}
 
-    # the dominant kernel: the longest of the three MFMA kernels
-    dominant = max(("forward", "backward_k_side", "backward_kprime_side"), key=lambda k: kernels[k]["ms"])
+    # ---- shader clock while the kernels run, and the peak it implies -------------------
+    bwd_call = lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2)
+    fwd_call = lambda: sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2)
+    clocks = {}
+    for cname, call, ms_call in (("forward", fwd_call, fwd_ms), ("backward", bwd_call, bwd_all_ms), ("step", step, ms_per_step)):
+        clocks[cname] = observed_clock_mhz(call, ms_call)
+    cus = props.multi_processor_count
+    peak_at = lambda mhz: cus * BF16_FLOP_PER_CLK_PER_CU * mhz * 1e6 / 1e12
+    clock = {"mhz": clocks, "method": "device cycle counter (60 ms spin kernel on a second stream) / event time",
+             "peak_bf16_tflops_at_observed_clock": {k: peak_at(v) for k, v in clocks.items()},
+             "published_peak_bf16_tflops": PEAK_BF16_TFLOPS,
+             "published_peak_is": "%d CU x 2400 MHz x %d flop/clk/CU" % (cus, BF16_FLOP_PER_CLK_PER_CU)}
+    kernels["forward"]["frac_at_observed_clock"] = kernels["forward"]["tflops"] / peak_at(clocks["forward"])
+    for name in ("backward_k_side", "backward_kprime_side", "backward"):
+        kernels[name]["frac_at_observed_clock"] = kernels[name]["tflops"] / peak_at(clocks["backward"])
+
+    # The dominant kernel: the K-side kernel is one launch, so its own duration is measured here
+    # (call with only dK, dV requested minus the row-dot kernel); the other two groups hold three
+    # launches each (their pre-pass and a short epilogue kernel beside the main one).
+    dominant = "backward_k_side"
+    longest_group = max(("forward", "backward_k_side", "backward_kprime_side"), key=lambda k: kernels[k]["ms"])
     roofline = {
         "bound": "mfma", "kernel": kernels[dominant]["kernel"],
         "achieved": kernels[dominant]["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
         "frac": kernels[dominant]["frac_bf16_peak"],
-        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dominant)),
+        "traffic": kernels[dominant]["traffic"],
         "algorithmic_flops_per_launch": kernels[dominant]["flops"],
         "avg_ms": kernels[dominant]["ms"],
+        "mfma_busy": kernels[dominant]["mfma_busy"],
+        "frac_at_observed_clock": kernels[dominant]["frac_at_observed_clock"],
+        "counters_from": key_sources.get(wl),
+        "longest_group": {"name": longest_group, "kernel": kernels[longest_group]["kernel"],
+                          "ms": kernels[longest_group]["ms"], "frac": kernels[longest_group]["frac_bf16_peak"]},
     }
     roofline_fwd = {
         "bound": "mfma", "kernel": kernels["forward"]["kernel"], "achieved": kernels["forward"]["tflops"],
         "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": kernels["forward"]["frac_bf16_peak"],
-        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "forward")),
+        "frac_at_observed_clock": kernels["forward"]["frac_at_observed_clock"],
+        "mfma_busy": kernels["forward"]["mfma_busy"], "traffic": kernels["forward"]["traffic"],
+        "counters_from": key_sources.get(wl),
         "hbm_gbs": kernels["forward"]["hbm_gbs"], "hbm_frac": kernels["forward"]["hbm_gbs"] / PEAK_HBM_GBS,
     }
 
@@ -235,15 +331,18 @@ def main():
         "config": {"workload": "%s: bf16 fwd+bwd B=%d H=%d N=%d D=%d w1=%d w2=%d scale=1/sqrt(D)" % (
                        args.workload, B, H, N, D, w1, w2),
                    "triples": T, "flops_fwd": fwd_flops, "flops_bwd": bwd_flops,
-                   "mfma_kernels": mfma, "device": props.name, "cus": props.multi_processor_count,
-                   "clock_mhz": props.clock_rate / 1e3 if hasattr(props, "clock_rate") else None},
+                   "mfma_kernels": mfma, "device": props.name, "cus": cus,
+                   "clock_mhz": clocks["step"]},
         "frac_bf16_peak": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
+        "frac_bf16_peak_at_observed_clock": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / peak_at(clocks["step"]),
+        "clock": clock,
         "roofline": roofline,
         "roofline_forward": roofline_fwd,
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_rows)
+        line["cpu_reference_literal"] = cpu_reference_literal(T // (B * H), "%s forward" % args.workload)
     print(json.dumps(line))
 
 
