@@ -44,6 +44,19 @@ def _rows(t):
     return t if ok else t.contiguous()
 
 
+def _pad_head_dim(D, dtype, flags):
+    """head_dim the kernels are run with.  The MFMA kernels start at head_dim 32 (one 32-column
+    value tile); 16-bit tensors with head_dim 16 are zero-padded to 32 on the way in (zero columns
+    add nothing to a logit and give zero output and gradient columns, which are dropped again), so
+    that they take the MFMA kernels instead of the fp32 FMA kernels.  The softmax scale is always
+    the caller's (1/sqrt(16) by default), not that of the padded width."""
+    return 32 if (D == 16 and dtype in (torch.bfloat16, torch.float16) and flags == _lib.FLAG_AUTO) else D
+
+
+def _padded(t, width):
+    return t if t.shape[-1] == width else torch.nn.functional.pad(t, (0, width - t.shape[-1]))
+
+
 def _strides(*tensors):
     return _lib.stride_array([(t.stride(0), t.stride(1), t.stride(2)) for t in tensors])
 
@@ -63,6 +76,11 @@ def simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bi
         scale = 1.0 / math.sqrt(D)
     if window_inclusive is None:
         window_inclusive = WINDOW_INCLUSIVE
+    width = _pad_head_dim(D, q.dtype, flags)
+    if width != D:
+        out, lse = simplicial_forward(*(_padded(t, width) for t in (q, k1, k2, v1, v2)), w1, w2, scale, k2_bias,
+                                      v2_bias, flags, window_inclusive)
+        return out[..., :D].contiguous(), lse
     q, k1, k2, v1, v2 = (_rows(t) for t in (q, k1, k2, v1, v2))
     with torch.cuda.device(q.device):
         out = torch.empty((B, N, H, D), dtype=q.dtype, device=q.device)
@@ -85,6 +103,11 @@ def simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2, scale=None, k
         scale = 1.0 / math.sqrt(D)
     if window_inclusive is None:
         window_inclusive = WINDOW_INCLUSIVE
+    width = _pad_head_dim(D, q.dtype, flags)
+    if width != D:
+        grads = simplicial_backward(*(_padded(t, width) for t in (q, k1, k2, v1, v2, out)), lse, _padded(dout, width),
+                                    w1, w2, scale, k2_bias, v2_bias, needs, flags, window_inclusive)
+        return tuple(g[..., :D].contiguous() if g is not None else None for g in grads)
     q, k1, k2, v1, v2, out, dout = (_rows(t) for t in (q, k1, k2, v1, v2, out, dout))
     dt = _DTYPES[q.dtype]
     reach1 = int(w1) if window_inclusive else int(w1) - 1

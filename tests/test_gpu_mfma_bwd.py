@@ -200,3 +200,28 @@ def test_packed_projection_views_take_the_mfma_kernels():
     want = oracle_all([c.cpu() for c in copies] + [dout.cpu()], w1, w2)
     assert_close_rel(out_v, want["out"], BF16_TOL, "out")
     assert_close_rel(grads_v[0], want["dq"], BF16_TOL, "dq")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_dim_16_is_padded_onto_the_mfma_kernels(dtype):
+    """head_dim 16 (simplicial/test_correctness.py:32): 16-bit tensors are zero-padded to 32 columns
+    by the host wrapper and run on the MFMA kernels; results equal those of the MFMA kernels on the
+    hand-padded tensors bit for bit (same scale) and meet the oracle at the 16-bit parity bar."""
+    import simplical_attn_amd as sa
+    B, N, H, D, w1, w2 = 2, 150, 3, 16, 40, 9
+    inp = make_inputs(B, N, H, D, seed=16, dtype=dtype)
+    got = run_device(inp, w1, w2, None, 0.1, -0.2, flags=0)
+    want = oracle_all(inp, w1, w2, None, 0.1, -0.2)
+    tol = BF16_TOL if dtype == torch.bfloat16 else 1e-2
+    for name in ("out", "lse") + GRADS:
+        assert got[name].shape[-1] == (N if name == "lse" else D)
+        assert_close_rel(got[name], want[name], tol, name)
+    dev = torch.device("cuda:0")
+    pad = [torch.nn.functional.pad(x.to(dev), (0, 16)) for x in inp]
+    out, lse = sa.simplicial_forward(*pad[:5], w1, w2, D ** -0.5, 0.1, -0.2, flags=MFMA)
+    grads = sa.simplicial_backward(*pad[:5], out, lse, pad[5], w1, w2, D ** -0.5, 0.1, -0.2, flags=MFMA)
+    assert torch.equal(got["out"], out[..., :D]) and torch.equal(got["lse"], lse)
+    assert not out[..., D:].any()
+    for name, g in zip(GRADS, grads):
+        assert torch.equal(got[name], g[..., :D]), name
+        assert not g[..., D:].any(), name
