@@ -122,6 +122,24 @@ def observed_clock_mhz(fn, ms_per_call, spin_ms=60.0):
     return cycles / e0.elapsed_time(e1) / 1e3
 
 
+def library_gemm_tflops(device, m=8192, iters=20):
+    """What the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) reaches on this device on N(0,1) operands and
+    on zeros, m x m x m: the matrix pipes draw more power on random operands than on quiet ones and the chip
+    slows down, so the published peak is out of reach for any kernel on the bench's data.  Context for the
+    roofline fractions, not a target and not part of the timed step."""
+    res = {}
+    c = torch.empty(m, m, device=device, dtype=torch.bfloat16)
+    for kind in ("zeros", "n01"):
+        a = torch.zeros(m, m, device=device, dtype=torch.bfloat16)
+        b = torch.zeros(m, m, device=device, dtype=torch.bfloat16)
+        if kind == "n01":
+            a.normal_()
+            b.normal_()
+        ms = time_gpu(lambda: torch.matmul(a, b.t(), out=c), iters, 5)
+        res[kind] = 2.0 * m ** 3 / ms / 1e9
+    return res
+
+
 def cpu_reference_literal(target_iterations, target_name):
     """The reference's literal triple loop (queries x K keys x K' keys, one weight at a time;
     simplicial/reference.py:39-74 as restated in oracle/) at configuration c1, the only one it
@@ -319,6 +337,13 @@ def main():
         "counters_from": key_sources.get(wl),
         "hbm_gbs": kernels["forward"]["hbm_gbs"], "hbm_frac": kernels["forward"]["hbm_gbs"] / PEAK_HBM_GBS,
     }
+
+    gemm = library_gemm_tflops(dev)
+    clock["library_gemm_bf16_tflops"] = {
+        "shape": "8192^3, torch.matmul", "n01_operands": gemm["n01"], "zero_operands": gemm["zeros"],
+        "n01_frac_of_published_peak": gemm["n01"] / PEAK_BF16_TFLOPS}
+    roofline["frac_of_library_gemm_on_n01"] = roofline["achieved"] / gemm["n01"]
+    roofline_fwd["frac_of_library_gemm_on_n01"] = roofline_fwd["achieved"] / gemm["n01"]
 
     line = {
         "metric": "fwd+bwd TFLOP/s & %% bf16 MFMA peak, N=%d D=%d w1=%d w2=%d" % (N, D, w1, w2),
