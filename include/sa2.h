@@ -68,7 +68,8 @@ const char* sa2_strerror(int status);
 /* 1 if sa2_forward would take the MFMA kernels for this problem under SA2_FLAG_AUTO
  * (given 16-byte aligned rows), 0 if it would take the generic kernels.  It answers for
  * the forward only: sa2_backward additionally falls back to the generic kernels for
- * fp16 or D = 32 problems whose K' window exceeds what its on-chip kernels hold. */
+ * D = 32 problems whose K' window exceeds what its on-chip kernels hold (several hundred
+ * positions). */
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype);
 
 /*

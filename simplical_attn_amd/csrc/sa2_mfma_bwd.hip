@@ -1,15 +1,15 @@
 // MFMA backward for gfx950: dispatch to the on-chip kernels (sa2_mfma_bwd_kp.hip for dQ, dK',
-// dV'; sa2_mfma_bwd_kv.hip for dK, dV; bf16 or fp16, head_dim 32, 64 or 128), and the bf16
-// workspace kernels (head_dim 64 or 128) that serve shapes whose K' window is too wide for them.
+// dV'; sa2_mfma_bwd_kv.hip for dK, dV; bf16 or fp16, head_dim 32, 64 or 128), and the workspace
+// kernels (bf16 or fp16, head_dim 64 or 128) that serve shapes whose K' window is too wide for them.
 //
 // Same expanded-row view as the forward: rows r = (i, delta), Q~[r] = q[i] *
-// k2~[i-delta] * scale*log2(e) and dO~[r] = dO[i] * v2~[i-delta], both bf16.  With
+// k2~[i-delta] * scale*log2(e) and dO~[r] = dO[i] * v2~[i-delta], both in the element type.  With
 // P = exp2(S - LSE*log2e) recomputed from the saved log-sum-exp and
 // dS = P * (dO~.v1 - D_i), the workspace kernels are:
 //
 //   row kernel      owns 32 queries x one delta per wavefront, sweeps the K window:
 //                   G[r,:] = scale * sum_j dS[r,j] k1[j,:]   and   R[r,:] = sum_j P[r,j] v1[j,:]
-//                   are written once per expanded row to a bf16 workspace;
+//                   are written once per expanded row to a 16-bit workspace;
 //   finalize        dQ[i]  = sum_delta G[(i,delta)] * k2~[i-delta]
 //                   dK'[k] = sum_delta G[(k+delta,delta)] * q[k+delta]
 //                   dV'[k] = sum_delta R[(k+delta,delta)] * dO[k+delta]
@@ -29,8 +29,8 @@ template <int D>
 struct RowCfg {
     static constexpr int DK = D / 16;
     static constexpr int DT = D / 32;
-    static constexpr int KS = D + 8;           // row-major tile row stride (bf16)
-    static constexpr int VS = TJ + 8;          // transposed tile row stride (bf16)
+    static constexpr int KS = D + 8;           // row-major tile row stride (elements)
+    static constexpr int VS = TJ + 8;          // transposed tile row stride (elements)
     static constexpr int RM_ELEMS = TJ * KS;
     static constexpr int TR_ELEMS = D * VS;
     static constexpr int STAGE = 2 * RM_ELEMS + 2 * TR_ELEMS;   // K, V row-major; K^T, V^T
@@ -40,7 +40,7 @@ struct RowCfg {
     static constexpr size_t LDS_BYTES = (size_t)2 * STAGE * 2;
 };
 
-// 4 rows x 2 columns of a [row][col] bf16 tile (one dword per row) -> two 8-byte
+// 4 rows x 2 columns of a [row][col] 16-bit tile (one dword per row) -> two 8-byte
 // groups of the transposed tile.
 __device__ __forceinline__ void transpose4x2(const uint32_t* x, uint2& lo, uint2& hi) {
     lo.x = (x[0] & 0xffffu) | (x[1] << 16);
@@ -49,9 +49,11 @@ __device__ __forceinline__ void transpose4x2(const uint32_t* x, uint2& lo, uint2
     hi.y = (x[2] >> 16) | (x[3] & 0xffff0000u);
 }
 
-template <int D>
+template <class E, int D>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ gws, uint16_t* __restrict__ rws) {
+    typedef typename E::scalar EL;
+    typedef typename E::x8 X8;
     using C = RowCfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* smem = (uint16_t*)smem_raw;
@@ -160,7 +162,7 @@ void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ g
             continue;
         }
 
-        bf16x8 qf[C::DK], dof[C::DK];
+        X8 qf[C::DK], dof[C::DK];
         floatx16 gacc[C::DT], racc[C::DT];
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
@@ -177,13 +179,13 @@ void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ g
             const uint4 vb = *(const uint4*)(v2p + (int64_t)k * p.v2.sn + col);
             const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w}, kw[4] = {kb.x, kb.y, kb.z, kb.w};
             const uint32_t dw[4] = {da.x, da.y, da.z, da.w}, vw[4] = {vb.x, vb.y, vb.z, vb.w};
-            bf16x8 r, d;
+            X8 r, d;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                r[2 * t] = (__bf16)(bf16_lo(qw[t]) * (bf16_lo(kw[t]) + p.k2_bias) * qscale);
-                r[2 * t + 1] = (__bf16)(bf16_hi(qw[t]) * (bf16_hi(kw[t]) + p.k2_bias) * qscale);
-                d[2 * t] = (__bf16)(bf16_lo(dw[t]) * (bf16_lo(vw[t]) + p.v2_bias));
-                d[2 * t + 1] = (__bf16)(bf16_hi(dw[t]) * (bf16_hi(vw[t]) + p.v2_bias));
+                r[2 * t] = (EL)(E::lo(qw[t]) * (E::lo(kw[t]) + p.k2_bias) * qscale);
+                r[2 * t + 1] = (EL)(E::hi(qw[t]) * (E::hi(kw[t]) + p.k2_bias) * qscale);
+                d[2 * t] = (EL)(E::lo(dw[t]) * (E::lo(vw[t]) + p.v2_bias));
+                d[2 * t + 1] = (EL)(E::hi(dw[t]) * (E::hi(vw[t]) + p.v2_bias));
             }
             qf[kk] = r;
             dof[kk] = d;
@@ -202,10 +204,10 @@ void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ g
             for (int v = 0; v < 16; ++v) sacc[v] = dpacc[v] = 0.f;
 #pragma unroll
             for (int kk = 0; kk < C::DK; ++kk) {
-                const bf16x8 ka = *(const bf16x8*)(Kr + ln * C::KS + kk * 16 + hf * 8);
-                const bf16x8 va = *(const bf16x8*)(Vr + ln * C::KS + kk * 16 + hf * 8);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], sacc, 0, 0, 0);
-                dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dpacc, 0, 0, 0);
+                const X8 ka = *(const X8*)(Kr + ln * C::KS + kk * 16 + hf * 8);
+                const X8 va = *(const X8*)(Vr + ln * C::KS + kk * 16 + hf * 8);
+                sacc = E::mfma(ka, qf[kk], sacc, 0, 0, 0);
+                dpacc = E::mfma(va, dof[kk], dpacc, 0, 0, 0);
             }
             float pv[16], dsv[16];
 #pragma unroll
@@ -224,22 +226,22 @@ void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ g
                 pv[v] = fast_exp2(pv[v]);
                 dsv[v] = pv[v] * (dpacc[v] - dsum);
             }
-            bf16x8 pb[2], dsb[2];
+            X8 pb[2], dsb[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    pb[ks][t] = (__bf16)pv[ks * 8 + t];
-                    dsb[ks][t] = (__bf16)dsv[ks * 8 + t];
+                    pb[ks][t] = (EL)pv[ks * 8 + t];
+                    dsb[ks][t] = (EL)dsv[ks * 8 + t];
                 }
 #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
-                    const bf16x8 kt = *(const bf16x8*)(Kt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
-                    const bf16x8 vt = *(const bf16x8*)(Vt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
-                    gacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt, dsb[ks], gacc[dt], 0, 0, 0);
-                    racc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pb[ks], racc[dt], 0, 0, 0);
+                    const X8 kt = *(const X8*)(Kt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                    const X8 vt = *(const X8*)(Vt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                    gacc[dt] = E::mfma(kt, dsb[ks], gacc[dt], 0, 0, 0);
+                    racc[dt] = E::mfma(vt, pb[ks], racc[dt], 0, 0, 0);
                 }
 
             if (g + 1 < total_steps) store_tile((g + 1) & 1);
@@ -254,11 +256,11 @@ void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ g
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
-                    union { __bf16 h[4]; uint2 u; } a, c;
+                    union { EL h[4]; uint2 u; } a, c;
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        a.h[t] = (__bf16)(gacc[dt][4 * g4 + t] * p.scale);
-                        c.h[t] = (__bf16)racc[dt][4 * g4 + t];
+                        a.h[t] = (EL)(gacc[dt][4 * g4 + t] * p.scale);
+                        c.h[t] = (EL)racc[dt][4 * g4 + t];
                     }
                     *(uint2*)(gws + base + dt * 32 + 8 * g4) = a.u;
                     *(uint2*)(rws + base + dt * 32 + 8 * g4) = c.u;
@@ -269,7 +271,7 @@ void mfma_bwd_row_kernel(Problem p, int nqb, int total, uint16_t* __restrict__ g
 
 // =============================================================== finalize ====
 // One wavefront per (batch, head, position n): lanes own column pairs.
-template <int D>
+template <class E, int D>
 __global__ __launch_bounds__(256) void mfma_bwd_finalize_kernel(Problem p, const uint16_t* __restrict__ gws,
                                                                const uint16_t* __restrict__ rws, int64_t rows) {
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -292,10 +294,10 @@ __global__ __launch_bounds__(256) void mfma_bwd_finalize_kernel(Problem p, const
         for (int dl = 0; dl <= dmax; ++dl) {
             const uint32_t gx = *(const uint32_t*)(gws + ((wrow + n) * nd + dl) * D + c2);
             const uint32_t kx = *(const uint32_t*)(k2p + (int64_t)(n - dl) * p.k2.sn);
-            a0 = fmaf(bf16_lo(gx), bf16_lo(kx) + p.k2_bias, a0);
-            a1 = fmaf(bf16_hi(gx), bf16_hi(kx) + p.k2_bias, a1);
+            a0 = fmaf(E::lo(gx), E::lo(kx) + p.k2_bias, a0);
+            a1 = fmaf(E::hi(gx), E::hi(kx) + p.k2_bias, a1);
         }
-        const uint32_t o = (uint32_t)f32_to_bf16_bits(a0) | ((uint32_t)f32_to_bf16_bits(a1) << 16);
+        const uint32_t o = E::pack(a0, a1);
         *(uint32_t*)((uint16_t*)p.dq.p + p.dq.off(b, n, h) + c2) = o;
     }
     if (p.dk2.p || p.dv2.p) {
@@ -308,17 +310,17 @@ __global__ __launch_bounds__(256) void mfma_bwd_finalize_kernel(Problem p, const
             const uint32_t rx = *(const uint32_t*)(rws + wo);
             const uint32_t qx = *(const uint32_t*)(qp + (int64_t)i * p.q.sn);
             const uint32_t dx = *(const uint32_t*)(dop + (int64_t)i * p.dout.sn);
-            k0 = fmaf(bf16_lo(gx), bf16_lo(qx), k0);
-            k1 = fmaf(bf16_hi(gx), bf16_hi(qx), k1);
-            v0 = fmaf(bf16_lo(rx), bf16_lo(dx), v0);
-            v1 = fmaf(bf16_hi(rx), bf16_hi(dx), v1);
+            k0 = fmaf(E::lo(gx), E::lo(qx), k0);
+            k1 = fmaf(E::hi(gx), E::hi(qx), k1);
+            v0 = fmaf(E::lo(rx), E::lo(dx), v0);
+            v1 = fmaf(E::hi(rx), E::hi(dx), v1);
         }
         if (p.dk2.p)
             *(uint32_t*)((uint16_t*)p.dk2.p + p.dk2.off(b, n, h) + c2) =
-                (uint32_t)f32_to_bf16_bits(k0) | ((uint32_t)f32_to_bf16_bits(k1) << 16);
+                E::pack(k0, k1);
         if (p.dv2.p)
             *(uint32_t*)((uint16_t*)p.dv2.p + p.dv2.off(b, n, h) + c2) =
-                (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+                E::pack(v0, v1);
     }
 }
 
@@ -329,8 +331,8 @@ template <int D>
 struct ColCfg {
     static constexpr int DK = D / 16;
     static constexpr int DT = D / 32;
-    static constexpr int KS = D + 8;           // row-major unit tile row stride (bf16)
-    static constexpr int VS = BQ + 8;          // transposed unit tile row stride (bf16)
+    static constexpr int KS = D + 8;           // row-major unit tile row stride (elements)
+    static constexpr int VS = BQ + 8;          // transposed unit tile row stride (elements)
     static constexpr int RM_ELEMS = BQ * KS;
     static constexpr int TR_ELEMS = D * VS;
     static constexpr int UNIT = 2 * RM_ELEMS + 2 * TR_ELEMS;    // Q~, dO~ row-major; Q~^T, dO~^T
@@ -342,9 +344,11 @@ struct ColCfg {
     static constexpr size_t LDS_BYTES = (size_t)(2 * UNIT + RAW) * 2 + 2 * BQ * sizeof(float);
 };
 
-template <int D>
+template <class E, int D>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void mfma_bwd_col_kernel(Problem p, int njb, int total) {
+    typedef typename E::scalar EL;
+    typedef typename E::x8 X8;
     using C = ColCfg<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* units = (uint16_t*)smem_raw;                 // two formed units
@@ -377,11 +381,11 @@ void mfma_bwd_col_kernel(Problem p, int njb, int total) {
     const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
 
     // K and V rows of this wavefront as resident MFMA B operands (column = K row)
-    bf16x8 kfr[C::DK], vfr[C::DK];
+    X8 kfr[C::DK], vfr[C::DK];
 #pragma unroll
     for (int kk = 0; kk < C::DK; ++kk) {
-        kfr[kk] = *(const bf16x8*)(k1p + (int64_t)jc * p.k1.sn + kk * 16 + hf * 8);
-        vfr[kk] = *(const bf16x8*)(v1p + (int64_t)jc * p.v1.sn + kk * 16 + hf * 8);
+        kfr[kk] = *(const X8*)(k1p + (int64_t)jc * p.k1.sn + kk * 16 + hf * 8);
+        vfr[kk] = *(const X8*)(v1p + (int64_t)jc * p.v1.sn + kk * 16 + hf * 8);
     }
     floatx16 dkacc[C::DT], dvacc[C::DT];
 #pragma unroll
@@ -463,13 +467,13 @@ void mfma_bwd_col_kernel(Problem p, int njb, int total) {
                         const uint32_t ka = *(const uint32_t*)(k2_s + kr * D + 2 * cp);
                         const uint32_t da = *(const uint32_t*)(do_s + r * D + 2 * cp);
                         const uint32_t va = *(const uint32_t*)(v2_s + kr * D + 2 * cp);
-                        const float q0 = bf16_lo(qa) * (bf16_lo(ka) + p.k2_bias) * qscale;
-                        const float q1 = bf16_hi(qa) * (bf16_hi(ka) + p.k2_bias) * qscale;
-                        const float d0 = bf16_lo(da) * (bf16_lo(va) + p.v2_bias);
-                        const float d1 = bf16_hi(da) * (bf16_hi(va) + p.v2_bias);
-                        union { __bf16 h[2]; uint32_t u; } qq, dd;
-                        qq.h[0] = (__bf16)q0; qq.h[1] = (__bf16)q1;
-                        dd.h[0] = (__bf16)d0; dd.h[1] = (__bf16)d1;
+                        const float q0 = E::lo(qa) * (E::lo(ka) + p.k2_bias) * qscale;
+                        const float q1 = E::hi(qa) * (E::hi(ka) + p.k2_bias) * qscale;
+                        const float d0 = E::lo(da) * (E::lo(va) + p.v2_bias);
+                        const float d1 = E::hi(da) * (E::hi(va) + p.v2_bias);
+                        union { EL h[2]; uint32_t u; } qq, dd;
+                        qq.h[0] = (EL)q0; qq.h[1] = (EL)q1;
+                        dd.h[0] = (EL)d0; dd.h[1] = (EL)d1;
                         qx[t] = qq.u;
                         dx[t] = dd.u;
                         *(uint32_t*)(Qr + r * C::KS + 2 * cp) = qq.u;
@@ -504,10 +508,10 @@ void mfma_bwd_col_kernel(Problem p, int njb, int total) {
                     for (int v = 0; v < 16; ++v) sacc[v] = dpacc[v] = 0.f;
 #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) {
-                        const bf16x8 qa = *(const bf16x8*)(Qr + ln * C::KS + kk * 16 + hf * 8);
-                        const bf16x8 da = *(const bf16x8*)(Dr + ln * C::KS + kk * 16 + hf * 8);
-                        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kfr[kk], sacc, 0, 0, 0);
-                        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vfr[kk], dpacc, 0, 0, 0);
+                        const X8 qa = *(const X8*)(Qr + ln * C::KS + kk * 16 + hf * 8);
+                        const X8 da = *(const X8*)(Dr + ln * C::KS + kk * 16 + hf * 8);
+                        sacc = E::mfma(qa, kfr[kk], sacc, 0, 0, 0);
+                        dpacc = E::mfma(da, vfr[kk], dpacc, 0, 0, 0);
                     }
                     float pv[16], dsv[16];
 #pragma unroll
@@ -530,23 +534,23 @@ void mfma_bwd_col_kernel(Problem p, int njb, int total) {
                         pv[v] = fast_exp2(pv[v]);
                         dsv[v] = pv[v] * (dpacc[v] - dsumr[v]);
                     }
-                    bf16x8 pb[2], dsb[2];
+                    X8 pb[2], dsb[2];
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
                         for (int t = 0; t < 8; ++t) {
-                            pb[ks][t] = (__bf16)pv[ks * 8 + t];
-                            dsb[ks][t] = (__bf16)dsv[ks * 8 + t];
+                            pb[ks][t] = (EL)pv[ks * 8 + t];
+                            dsb[ks][t] = (EL)dsv[ks * 8 + t];
                         }
                     // dV^T[d, j] += dO~^T[d, r] P[r, j];  dK^T[d, j] += Q~^T[d, r] dS[r, j]
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) {
-                            const bf16x8 dta = *(const bf16x8*)(Dt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
-                            const bf16x8 qta = *(const bf16x8*)(Qt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
-                            dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dta, pb[ks], dvacc[dt], 0, 0, 0);
-                            dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qta, dsb[ks], dkacc[dt], 0, 0, 0);
+                            const X8 dta = *(const X8*)(Dt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                            const X8 qta = *(const X8*)(Qt + (dt * 32 + ln) * C::VS + ks * 16 + hf * 8);
+                            dvacc[dt] = E::mfma(dta, pb[ks], dvacc[dt], 0, 0, 0);
+                            dkacc[dt] = E::mfma(qta, dsb[ks], dkacc[dt], 0, 0, 0);
                         }
                 }
                 __syncthreads();
@@ -561,11 +565,11 @@ void mfma_bwd_col_kernel(Problem p, int njb, int total) {
         for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
-                union { __bf16 h[4]; uint2 u; } a, c;
+                union { EL h[4]; uint2 u; } a, c;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    a.h[t] = (__bf16)(dkacc[dt][4 * g4 + t] * LN2);     // Q~ carries scale*log2(e)
-                    c.h[t] = (__bf16)dvacc[dt][4 * g4 + t];
+                    a.h[t] = (EL)(dkacc[dt][4 * g4 + t] * LN2);     // Q~ carries scale*log2(e)
+                    c.h[t] = (EL)dvacc[dt][4 * g4 + t];
                 }
                 if (dkp) *(uint2*)(dkp + dt * 32 + 8 * g4) = a.u;
                 if (dvp) *(uint2*)(dvp + dt * 32 + 8 * g4) = c.u;
@@ -573,14 +577,14 @@ void mfma_bwd_col_kernel(Problem p, int njb, int total) {
     }
 }
 
-template <int D>
+template <class E, int D>
 int launch_col_part(const Problem& p, hipStream_t st) {
     using C = ColCfg<D>;
     const int njb = (p.N + CJ - 1) / CJ;
     const int64_t total = (int64_t)njb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-    if (!allow_full_lds((const void*)mfma_bwd_col_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL(mfma_bwd_col_kernel<D>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, njb,
+    if (!allow_full_lds((const void*)mfma_bwd_col_kernel<E, D>)) return SA2_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL((mfma_bwd_col_kernel<E, D>), dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, njb,
                        (int)total);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
@@ -589,7 +593,7 @@ size_t expanded_ws_bytes(int B, int N, int H, int D, int w2) {
     return (size_t)B * H * N * (size_t)(w2 + 1) * D * sizeof(uint16_t);
 }
 
-template <int D>
+template <class E, int D>
 int launch_row_part(const Problem& p, hipStream_t st) {
     using C = RowCfg<D>;
     const int nqb = (p.N + BQ - 1) / BQ;
@@ -599,12 +603,12 @@ int launch_row_part(const Problem& p, hipStream_t st) {
     if (p.scratch_bytes < 2 * one) return SA2_ERR_WORKSPACE_TOO_SMALL;
     uint16_t* gws = (uint16_t*)p.scratch;
     uint16_t* rws = (uint16_t*)((char*)p.scratch + one);
-    if (!allow_full_lds((const void*)mfma_bwd_row_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL(mfma_bwd_row_kernel<D>, dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, nqb,
+    if (!allow_full_lds((const void*)mfma_bwd_row_kernel<E, D>)) return SA2_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL((mfma_bwd_row_kernel<E, D>), dim3((unsigned)total), dim3(NTHREADS), C::LDS_BYTES, st, p, nqb,
                        (int)total, gws, rws);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     const int64_t rows = (int64_t)p.B * p.H * p.N;
-    hipLaunchKernelGGL(mfma_bwd_finalize_kernel<D>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, p, gws, rws,
+    hipLaunchKernelGGL((mfma_bwd_finalize_kernel<E, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, p, gws, rws,
                        rows);
     return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
 }
@@ -613,8 +617,8 @@ int launch_row_part(const Problem& p, hipStream_t st) {
 
 bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
     if (!mfma_supported(B, N, H, D, w1, w2, dtype)) return false;
-    // the workspace fallback kernels for wide K' windows exist for bf16 with D = 64 or 128 only
-    return (dtype == SA2_BF16 && D != 32) || (kp_fits(D, w2) && kv_fits(D, w2));
+    // the workspace kernels for wide K' windows exist for D = 64 and 128
+    return D != 32 || (kp_fits(D, w2) && kv_fits(D, w2));
 }
 
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
@@ -629,12 +633,14 @@ int launch_mfma_bwd(const Problem& p, int dtype, hipStream_t st) {
     if (rc != SA2_OK) return rc;
     if (p.dq.p || p.dk2.p || p.dv2.p) {
         if (kp_fits(p.D, p.w2)) rc = launch_mfma_bwd_kp(p, dtype, st);
-        else rc = p.D == 128 ? launch_row_part<128>(p, st) : launch_row_part<64>(p, st);
+        else if (dtype == SA2_F16) rc = p.D == 128 ? launch_row_part<ElemF16, 128>(p, st) : launch_row_part<ElemF16, 64>(p, st);
+        else rc = p.D == 128 ? launch_row_part<ElemBF16, 128>(p, st) : launch_row_part<ElemBF16, 64>(p, st);
         if (rc != SA2_OK) return rc;
     }
     if (p.dk1.p || p.dv1.p) {
         if (kv_fits(p.D, p.w2)) rc = launch_mfma_bwd_kv(p, dtype, st);
-        else rc = p.D == 128 ? launch_col_part<128>(p, st) : launch_col_part<64>(p, st);
+        else if (dtype == SA2_F16) rc = p.D == 128 ? launch_col_part<ElemF16, 128>(p, st) : launch_col_part<ElemF16, 64>(p, st);
+        else rc = p.D == 128 ? launch_col_part<ElemBF16, 128>(p, st) : launch_col_part<ElemBF16, 64>(p, st);
     }
     return rc;
 }

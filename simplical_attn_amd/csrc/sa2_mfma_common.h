@@ -36,6 +36,12 @@ struct ElemBF16 {
     static constexpr float WEIGHT_LIMIT = 1.0e30f;
     static __device__ __forceinline__ float lo(uint32_t x) { return __uint_as_float(x << 16); }
     static __device__ __forceinline__ float hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        union { __bf16 h[2]; uint32_t u; } v;
+        v.h[0] = (__bf16)a;
+        v.h[1] = (__bf16)b;
+        return v.u;
+    }
     static __device__ __forceinline__ floatx16 mfma(x8 a, x8 b, floatx16 c, int, int, int) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
@@ -58,6 +64,12 @@ struct ElemF16 {
         union { uint32_t u; _Float16 h[2]; } v;
         v.u = x;
         return (float)v.h[1];
+    }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        union { _Float16 h[2]; uint32_t u; } v;
+        v.h[0] = (_Float16)a;
+        v.h[1] = (_Float16)b;
+        return v.u;
     }
     static __device__ __forceinline__ floatx16 mfma(x8 a, x8 b, floatx16 c, int, int, int) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);

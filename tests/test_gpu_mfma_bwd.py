@@ -50,17 +50,24 @@ def test_small_shapes_vs_oracle(case):
             assert_close_rel(got[name], want[name], BF16_TOL, name, label="small shapes bf16 (bwd)")
 
 
-@pytest.mark.parametrize("case", [SMALL[1], SMALL[6], (1, 300, 2, 64, 96, 16, 0.1, 0.0), (2, 160, 2, 128, 64, 33, 0.0, 0.0)])
+@pytest.mark.parametrize("case", [SMALL[1], SMALL[6], (1, 300, 2, 64, 96, 16, 0.1, 0.0), (2, 160, 2, 128, 64, 33, 0.0, 0.0),
+                                  SMALL[12], SMALL[13],                  # workspace kernels
+                                  (1, 400, 1, 64, 24, 330, 0.0, 0.1)])   # the same at head_dim 64
 def test_small_shapes_fp16_vs_oracle(case):
-    """fp16 elements on the same kernels (fp16 MFMA).  Tolerance: max|diff| <= 1e-2 * max|ref| per
-    tensor (P, dS and the row-dot D are rounded to fp16 inside the kernels)."""
+    """fp16 elements on the same kernels (fp16 MFMA), the workspace kernels for wide K' windows included.
+    Tolerance: max|diff| <= 1.5e-2 * max|ref| per tensor.  The products q*k2~ and dO*v2~ are rounded to
+    fp16 before the MFMAs, as the reference rounds its products to the GEMM type (kernels.py:106,
+    301-302); over most of a tensor that costs 1e-3, but on the first query rows, whose windows hold
+    a few triples, the weights do not average it out: the worst measured element is dk1 at position 1
+    of the biased w2 = 100 case, 1.22e-2 (the same on the on-chip kernels at w2 = 60; the fp32
+    kernels, which do not round the products, measure 1.8e-3 there)."""
     B, N, H, D, w1, w2, kb, vb = case
     inp = make_inputs(B, N, H, D, seed=N + D + w1, dtype=torch.float16)
     got = run_device(inp, w1, w2, None, kb, vb, flags=MFMA)
     want = oracle_all(inp, w1, w2, None, kb, vb)
     for name in GRADS:
         assert got[name].dtype == torch.float16
-        assert_close_rel(got[name], want[name], 1e-2, name, label="small shapes fp16 (bwd)")
+        assert_close_rel(got[name], want[name], 1.5e-2, name, label="small shapes fp16 (bwd)")
 
 
 def check_rows(got, inp, w1, w2, rows, label=None):
