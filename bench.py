@@ -260,6 +260,24 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ms_per_step = e0.elapsed_time(e1) / args.steps
 
+    # ---- the forward's and the backward's share of a step (events inside further steps) ----
+    # Back-to-back forwards draw more power than the step's mix; on some boxes the forward runs up
+    # to 5 % faster between two backwards than in a loop of its own.  Both figures are reported.
+    marks = []
+    for _ in range(max(5, args.steps)):
+        for t in leaves:
+            t.grad = None
+        m = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        m[0].record()
+        o = attn(*leaves)
+        m[1].record()
+        o.backward(dout)
+        m[2].record()
+        marks.append(m)
+    torch.cuda.synchronize()
+    fwd_in_step_ms = sum(m[0].elapsed_time(m[1]) for m in marks) / len(marks)
+    bwd_in_step_ms = sum(m[1].elapsed_time(m[2]) for m in marks) / len(marks)
+
     # ---- per-kernel-group durations (same stream, events) -------------------
     out, lse = sa.simplicial_forward(q, k1, k2, v1, v2, w1, w2)
     ksteps = max(5, args.steps)
@@ -291,8 +309,11 @@ def main():
         k["mfma_busy"] = keys.get((wl, name, "mfma_busy"))          # rocprofv3, from profiles/
         k["traffic"] = keys.get((wl, name, "traffic_bytes"))
     kernels["forward"]["hbm_gbs"] = fwd_bytes / fwd_ms / 1e6
+    kernels["forward"]["ms_in_step"] = fwd_in_step_ms
+    kernels["forward"]["frac_bf16_peak_in_step"] = fwd_flops / fwd_in_step_ms / 1e9 / PEAK_BF16_TFLOPS
     kernels["backward"] = {"ms": bwd_all_ms, "tflops": bwd_flops / bwd_all_ms / 1e9, "hbm_gbs": bwd_bytes / bwd_all_ms / 1e6,
                            "frac_bf16_peak": bwd_flops / bwd_all_ms / 1e9 / PEAK_BF16_TFLOPS}
+    kernels["backward"]["ms_in_step"] = bwd_in_step_ms
     kernels["rowdot"] = {"ms": rowdot_ms, "hbm_gbs": (4 * E + 4 * B * H * N) / rowdot_ms / 1e6}
 
     # ---- shader clock while the kernels run, and the peak it implies -------------------
@@ -336,6 +357,8 @@ def main():
         "mfma_busy": kernels["forward"]["mfma_busy"], "traffic": kernels["forward"]["traffic"],
         "counters_from": key_sources.get(wl),
         "hbm_gbs": kernels["forward"]["hbm_gbs"], "hbm_frac": kernels["forward"]["hbm_gbs"] / PEAK_HBM_GBS,
+        "avg_ms": fwd_ms, "ms_in_step": fwd_in_step_ms,
+        "frac_in_step": kernels["forward"]["frac_bf16_peak_in_step"],
     }
 
     gemm = library_gemm_tflops(dev)
