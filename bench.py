@@ -137,7 +137,62 @@ def library_gemm_tflops(device, m=8192, iters=20):
             b.normal_()
         ms = time_gpu(lambda: torch.matmul(a, b.t(), out=c), iters, 5)
         res[kind] = 2.0 * m ** 3 / ms / 1e9
+        pw = power_under(lambda: torch.matmul(a, b.t(), out=c), 0.6)
+        if pw is not None:
+            pw["pj_per_flop"] = pw["joules_per_call"] / (2.0 * m ** 3) * 1e12
+        res[kind + "_power"] = pw
     return res
+
+
+POWER_GLOB = "/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"
+
+
+def board_power_w():
+    """Board power in watts from the amdgpu hwmon node of the first card (None where it cannot be read)."""
+    import glob
+    for path in sorted(glob.glob(POWER_GLOB)):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError):
+            continue
+    return None
+
+
+def board_power_cap_w():
+    import glob
+    for path in sorted(glob.glob(POWER_GLOB.replace("power1_input", "power1_cap"))):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError):
+            continue
+    return None
+
+
+def power_under(fn, seconds=0.8):
+    """Average board power while `fn` runs back to back for `seconds` (sampled between batches of
+    calls during the second half), with the average duration of a call in that loop."""
+    if board_power_w() is None:
+        return None
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    calls, samples = 0, []
+    while True:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        calls += 10
+        elapsed = time.perf_counter() - t0
+        if elapsed > 0.5 * seconds:
+            samples.append(board_power_w())
+        if elapsed > seconds:
+            break
+    watts = sum(samples) / len(samples)
+    ms = elapsed / calls * 1e3
+    return {"watts": watts, "ms_per_call": ms, "joules_per_call": watts * ms * 1e-3}
 
 
 def cpu_reference_literal(target_iterations, target_name):
@@ -361,10 +416,20 @@ def main():
         "frac_in_step": kernels["forward"]["frac_bf16_peak_in_step"],
     }
 
+    # ---- board power: these kernels run at the board's power limit on N(0,1) data ----------
+    idle_w = board_power_w()
+    power = None
+    if idle_w is not None:
+        power = {"source": POWER_GLOB, "cap_w": board_power_cap_w(),
+                 "step": power_under(step), "forward": power_under(fwd_call), "backward": power_under(bwd_call)}
+        power["forward"]["pj_per_algorithmic_flop"] = power["forward"]["joules_per_call"] / fwd_flops * 1e12
+        power["backward"]["pj_per_algorithmic_flop"] = power["backward"]["joules_per_call"] / bwd_flops * 1e12
+        power["step"]["pj_per_algorithmic_flop"] = power["step"]["joules_per_call"] / (fwd_flops + bwd_flops) * 1e12
     gemm = library_gemm_tflops(dev)
     clock["library_gemm_bf16_tflops"] = {
         "shape": "8192^3, torch.matmul", "n01_operands": gemm["n01"], "zero_operands": gemm["zeros"],
-        "n01_frac_of_published_peak": gemm["n01"] / PEAK_BF16_TFLOPS}
+        "n01_frac_of_published_peak": gemm["n01"] / PEAK_BF16_TFLOPS,
+        "n01_power": gemm["n01_power"], "zero_power": gemm["zeros_power"]}
     roofline["frac_of_library_gemm_on_n01"] = roofline["achieved"] / gemm["n01"]
     roofline_fwd["frac_of_library_gemm_on_n01"] = roofline_fwd["achieved"] / gemm["n01"]
 
@@ -384,6 +449,7 @@ def main():
         "frac_bf16_peak": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
         "frac_bf16_peak_at_observed_clock": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / peak_at(clocks["step"]),
         "clock": clock,
+        "power": power,
         "roofline": roofline,
         "roofline_forward": roofline_fwd,
         "kernels": kernels,
