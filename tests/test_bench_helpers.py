@@ -52,3 +52,12 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode == 2
     assert "one GPU" in res.stderr and not res.stdout.strip()
+
+
+def test_board_power_reads_a_number_or_nothing():
+    w = bench.board_power_w()
+    assert w is None or 0 < w < 5000
+    cap = bench.board_power_cap_w()
+    assert cap is None or cap > 0
+    if w is None:
+        assert bench.power_under(lambda: None) is None
