@@ -9,7 +9,8 @@
 //       through LDS and accumulates dV^T += dO~^T.P;
 //   the "dS" wavefront computes dP = dO~.V^T - D and, one unit behind, dS = P*dP and
 //       dK^T += Q~^T.dS.
-// Transposed operands come from the row-major unit tiles through ds_read_b64_tr_b16.
+// Transposed operands come from the same unit tiles through ds_read_b64_tr_b16; the tiles are laid
+// out in row groups so that both kinds of read are free of bank conflicts.
 // Every output element has one writer and a fixed summation order.
 #include <type_traits>
 
@@ -27,16 +28,21 @@ template <int D>
 struct KvCfg {
     static constexpr int DK = D / 16;
     static constexpr int DT = D / 32;
-    static constexpr int TS = D + 24;          // unit tile row stride (bf16)
-    static constexpr int TILE = BQ * TS;
-    static constexpr int UNIT = 2 * TILE;      // Q~ tile, then dO~ tile
+    // A unit tile (32 rows) in LDS keeps groups of RPW rows together: within a group the 16-byte
+    // chunk c of row q sits at byte (c * RPW + q) * 16, groups lie GROUP bytes apart.  Row operand
+    // reads (16 bytes per lane) and transposed operand reads are both bank-conflict free in it.
+    static constexpr int RPW = 512 / D;        // rows per group: 4 (D = 128), 8 (D = 64), 16 (D = 32)
+    static constexpr int GROUP = 1024 + 16 * RPW;
+    static constexpr int TILE_BYTES = (BQ / RPW) * GROUP;
+    static constexpr int UNIT_BYTES = 2 * TILE_BYTES;      // Q~ tile, then dO~ tile
+    static constexpr int row_off(int r) { return (r / RPW) * GROUP + (r % RPW) * 16; }    // chunk 0 of row r
     static constexpr int NUNIT = 3;
-    static constexpr int RS = D + 8;           // K'/V' row stride (bf16)
-    static constexpr int FS = D + 4;           // q / dO row stride (fp32)
+    static constexpr int RS = D + D / 4;       // K'/V' row stride (bf16): the forming threads' reads (RPW rows x 16 bytes per 16 lanes) hit distinct banks
+    static constexpr int FS = D;               // q / dO row stride (fp32); read once per query block, unpadded
     static constexpr int PX_BYTES = VPAIR * 2 * 64 * 32;
     static constexpr size_t LDS_LIMIT = 160 * 1024;
     static size_t lds_bytes(int w2) {
-        return (size_t)NUNIT * UNIT * 2 + PX_BYTES + 2 * BQ * FS * 4 + 2 * (size_t)(BQ + w2) * RS * 2 + 4 * BQ * 4;
+        return (size_t)NUNIT * UNIT_BYTES + PX_BYTES + 2 * BQ * FS * 4 + 2 * (size_t)(BQ + w2) * RS * 2 + 4 * BQ * 4;
     }
     static bool fits(int w2) { return lds_bytes(w2) <= LDS_LIMIT; }
 };
@@ -51,8 +57,8 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int SR = BQ + w2;                                   // K'/V' rows kept per query block
-    uint16_t* units = (uint16_t*)smem_raw;
-    unsigned char* px = smem_raw + (size_t)C::NUNIT * C::UNIT * 2;
+    unsigned char* units = smem_raw;
+    unsigned char* px = smem_raw + (size_t)C::NUNIT * C::UNIT_BYTES;
     float* q_s = (float*)(px + C::PX_BYTES);                  // [BQ][FS] q * scale*log2(e), fp32
     float* do_s = q_s + BQ * C::FS;                           // [BQ][FS] dO, fp32
     uint16_t* k2_s = (uint16_t*)(do_s + BQ * C::FS);          // [SR][RS] rows i0-w2 .. i0+31
@@ -138,19 +144,21 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     float qv[8], dv[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t) qv[t] = dv[t] = 0.f;
+    // Wavefront g < 32 / RPW forms row group g of a unit: lane L the 16-byte chunk L / RPW of row
+    // L % RPW, so that a wavefront's stores fill the group's 1 KB contiguously.
+    const bool former = wave < BQ / C::RPW;
+    const int f_row = wave * C::RPW + lane % C::RPW, f_col = lane / C::RPW;
     auto fetch_qd = [&]() {
-        constexpr int CPR = D / 8;
-        if (tid >= BQ * CPR) return;
-        const int row = tid / CPR, col = tid - row * CPR;
+        if (!former) return;
+        const int row = f_row, col = f_col;
         const float4 q0 = *(const float4*)(q_s + row * C::FS + col * 8), q1 = *(const float4*)(q_s + row * C::FS + col * 8 + 4);
         const float4 d0 = *(const float4*)(do_s + row * C::FS + col * 8), d1 = *(const float4*)(do_s + row * C::FS + col * 8 + 4);
         qv[0] = q0.x; qv[1] = q0.y; qv[2] = q0.z; qv[3] = q0.w; qv[4] = q1.x; qv[5] = q1.y; qv[6] = q1.z; qv[7] = q1.w;
         dv[0] = d0.x; dv[1] = d0.y; dv[2] = d0.z; dv[3] = d0.w; dv[4] = d1.x; dv[5] = d1.y; dv[6] = d1.z; dv[7] = d1.w;
     };
     auto form = [&](int delta, int slot) {
-        constexpr int CPR = D / 8;
-        if (tid >= BQ * CPR) return;
-        const int row = tid / CPR, col = tid - row * CPR;
+        if (!former) return;
+        const int row = f_row, col = f_col;
         const int kr = row - delta + w2;
         const uint4 kx = *(const uint4*)(k2_s + kr * C::RS + col * 8);
         const uint4 vx = *(const uint4*)(v2_s + kr * C::RS + col * 8);
@@ -171,15 +179,18 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                 d[2 * t + 1] = (EL)(dv[2 * t + 1] * E::hi(vw[t]));
             }
         }
-        uint16_t* dst = units + slot * C::UNIT + row * C::TS + col * 8;
+        unsigned char* dst = units + slot * C::UNIT_BYTES + wave * C::GROUP + lane * 16;
         *(X8*)dst = r;
-        *(X8*)(dst + C::TILE) = d;
+        *(X8*)(dst + C::TILE_BYTES) = d;
     };
 
     const uint32_t units_addr = lds_address(units);
     const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * 64 * 32 + lane * 32);
-    const uint32_t row_lane = (uint32_t)(ln * C::TS + hf * 8) * 2u;
-    const uint32_t col_lane = lds_column_lane_offset(C::TS, lane);
+    // this lane's part of a row operand read (row ln, the k-slots of its half; k-step kk adds
+    // kk * KKB) and of a transposed operand read (32-column block dt adds dt * DTB)
+    const uint32_t row_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);
+    const uint32_t col_lane = lds_group_column_lane_offset<C::RPW, C::GROUP>(lane);
+    constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;
 
     // ---- prologue: first block's raw rows, first unit --------------------------------
     load_raw(ib_lo);
@@ -207,12 +218,12 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             typedef const X8 __attribute__((address_space(3)))* lds_b8;
             const uint32_t a = px_addr + (uint32_t)((pstep & 1) * 64 * 32);
             const X8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
-            const uint32_t qt_addr = units_addr + (uint32_t)(pslot * C::UNIT) * 2u + col_lane;
+            const uint32_t qt_addr = units_addr + (uint32_t)(pslot * C::UNIT_BYTES) + col_lane;
             X8 qt[C::DT][2];
     #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) qt[dt][ks] = lds_column_operand_at<C::TS, X8>(qt_addr + dt * 64, ks);
+                for (int ks = 0; ks < 2; ++ks) qt[dt][ks] = lds_group_column_operand_at<C, X8>(qt_addr + dt * DTB, ks);
             X8 dsb[2];
     #pragma unroll
             for (int t = 0; t < 8; ++t) {
@@ -239,12 +250,12 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                 }
                 cur_ib = ib;
             }
-            const uint32_t u_addr = units_addr + (uint32_t)(slot * C::UNIT) * 2u;
+            const uint32_t u_addr = units_addr + (uint32_t)(slot * C::UNIT_BYTES);
             if (ROLE == 0) {
                 if (act) {
                     X8 qa[C::DK];
     #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) qa[kk] = lds_read_x8<X8>(u_addr + row_lane + kk * 32);
+                    for (int kk = 0; kk < C::DK; ++kk) qa[kk] = lds_read_x8<X8>(u_addr + row_lane + kk * KKB);
                     floatx16 sh;
                     const bool interior = (i0 >= jw + 31) && ((int64_t)i0 + 31 <= (int64_t)jw + w1) && (i0 + BQ - 1 < N) &&
                                           (i0 >= delta);
@@ -278,12 +289,12 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                         *(lds_b8)(uintptr_t)a = pb[0];
                         *(lds_b8)(uintptr_t)(a + 16) = pb[1];
                     }
-                    const uint32_t dt_addr = u_addr + (uint32_t)C::TILE * 2u + col_lane;
+                    const uint32_t dt_addr = u_addr + (uint32_t)C::TILE_BYTES + col_lane;
                     X8 da[C::DT][2];
     #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
-                        for (int ks = 0; ks < 2; ++ks) da[dt][ks] = lds_column_operand_at<C::TS, X8>(dt_addr + dt * 64, ks);
+                        for (int ks = 0; ks < 2; ++ks) da[dt][ks] = lds_group_column_operand_at<C, X8>(dt_addr + dt * DTB, ks);
     #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
@@ -294,10 +305,10 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
                 // first the previous unit (its dP is still in dp_prev), then this unit's dP
                 if (act_prev) consume(slot == 0 ? C::NUNIT - 1 : slot - 1, step - 1);
                 if (act) {
-                    const uint32_t d_addr = u_addr + (uint32_t)C::TILE * 2u;
+                    const uint32_t d_addr = u_addr + (uint32_t)C::TILE_BYTES;
                     X8 da[C::DK];
     #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) da[kk] = lds_read_x8<X8>(d_addr + row_lane + kk * 32);
+                    for (int kk = 0; kk < C::DK; ++kk) da[kk] = lds_read_x8<X8>(d_addr + row_lane + kk * KKB);
                     dp_prev = E::mfma(da[0], kvf[0], negr, 0, 0, 0);
     #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)

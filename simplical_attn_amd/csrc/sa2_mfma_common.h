@@ -126,6 +126,20 @@ __device__ __forceinline__ uint32_t lds_group_column_lane_offset(int lane) {
     const int cc = 16 * (grp & 1) + 4 * (s & 3);         // column within the 32-column block
     return (uint32_t)((rr / RPW) * GROUP + ((cc / 8) * RPW + rr % RPW) * 16 + (cc % 8) * 2);
 }
+// The operand itself (compiler-visible reads): `addr` = tile + lane part + block * 64 * RPW; k-step ks
+// takes rows 16*ks .. 16*ks+15.  CFG supplies row_off(r), the byte offset of row r.
+template <class CFG, class X8 = bf16x8>
+__device__ __forceinline__ X8 lds_group_column_operand_at(uint32_t addr, int ks) {
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef v4s __attribute__((address_space(3)))* lds_v4s;
+    const uint32_t o0 = ks ? (uint32_t)CFG::row_off(16) : 0u, o1 = ks ? (uint32_t)CFG::row_off(24) : (uint32_t)CFG::row_off(8);
+    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + o0));
+    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + o1));
+    union { v4s h[2]; X8 v; } u;
+    u.h[0] = a;
+    u.h[1] = b;
+    return u.v;
+}
 // The same operand read in two phases for loops that keep direct global->LDS loads in
 // flight: the compiler would wait for every outstanding vector-memory operation before a
 // transpose-read builtin, so the reads are issued as opaque instructions and the wait for
