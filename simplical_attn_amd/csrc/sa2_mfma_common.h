@@ -87,38 +87,21 @@ __device__ __forceinline__ float other_half(float x) {
     return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
 }
 
-// Eight 16-bit elements of one COLUMN of a row-major [row][col] tile in LDS, as the A/B operand
-// of a 32x32x16 MFMA whose contraction index runs over the tile's rows, for the tile's
-// 32x32 sub-block at rows r0.., columns c0.. (`stride` = row stride in elements).  Lane l gets column c0 + l%32 and, for its half h = l/32, the rows
-//   r0 + 16*ks + 4*h + {0,1,2,3}   and   r0 + 16*ks + 8 + 4*h + {0,1,2,3}
-// which is exactly the k-slot order in which a 32x32 accumulator tile (rows = those rows)
-// hands its values to the other operand.  Uses the LDS transpose read: within 16 lanes,
-// lane s supplies the address of row s/4, columns 4*(s%4)..+3, and lane i receives
-// column i of those four rows.
-// The operand is read from LDS byte addresses.  lds_column_lane_offset() is the per-lane part
-// (bytes, for ks = 0, relative to the 32x32 sub-block); lds_column_operand_at() takes the sum of
-// the sub-block's LDS byte address and that lane part, so that inside a loop the address is one
-// add and everything else sits in the instructions' immediate offsets.
-__device__ __forceinline__ uint32_t lds_column_lane_offset(int stride, int lane) {
-    const int grp = lane >> 4, s = lane & 15;
-    return (uint32_t)(((4 * (grp >> 1) + (s >> 2)) * stride + 16 * (grp & 1) + 4 * (s & 3)) * 2);
-}
-template <int STRIDE, class X8 = bf16x8>
-__device__ __forceinline__ X8 lds_column_operand_at(uint32_t addr, int ks) {
-    typedef short v4s __attribute__((ext_vector_type(4)));
-    typedef v4s __attribute__((address_space(3)))* lds_v4s;
-    const v4s a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)(16 * ks * STRIDE * 2)));
-    const v4s b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(uintptr_t)(addr + (uint32_t)((16 * ks + 8) * STRIDE * 2)));
-    union { v4s h[2]; X8 v; } u;
-    u.h[0] = a;
-    u.h[1] = b;
-    return u.v;
-}
-// Tiles written by direct global->LDS loads keep groups of RPW rows together: within a group
-// the 16-byte chunk c of row q sits at byte (c * RPW + q) * 16, groups lie GROUP bytes apart.
-// Transposed MFMA operand out of such a tile (same lanes and k-slot order as
-// lds_column_operand_at): the lane part of the address, and the two reads of k-step ks of the
-// 32-column block whose byte address (block * 64 * RPW) is already in `addr`.
+// Tiles in LDS (written by direct global->LDS loads, or by wavefronts in the same order) keep
+// groups of RPW rows together: within a group the 16-byte chunk c of row q sits at byte
+// (c * RPW + q) * 16, groups lie GROUP bytes apart.  Row operand reads (16 bytes per lane) and the
+// transposed reads below are both free of bank conflicts in this layout.
+//
+// Transposed MFMA operand out of such a tile: eight 16-bit elements of one COLUMN of the tile, as
+// the A/B operand of a 32x32x16 MFMA whose contraction index runs over the tile's rows.  For a
+// 32-column block, lane l gets column l%32 and, for its half h = l/32, the rows
+//   16*ks + 4*h + {0,1,2,3}   and   16*ks + 8 + 4*h + {0,1,2,3}
+// which is exactly the k-slot order in which a 32x32 accumulator tile (rows = those rows) hands
+// its values to the other operand.  Uses the LDS transpose read: within 16 lanes, lane s supplies
+// the address of row s/4, columns 4*(s%4)..+3, and lane i receives column i of those four rows.
+// lds_group_column_lane_offset() is the lane part of the address (bytes, for ks = 0); the reads
+// take the sum of the tile's LDS byte address, the block's offset (block * 64 * RPW) and that lane
+// part, so that inside a loop the address is one add and everything else sits in immediate offsets.
 template <int RPW, int GROUP>
 __device__ __forceinline__ uint32_t lds_group_column_lane_offset(int lane) {
     const int grp = lane >> 4, s = lane & 15;
