@@ -136,6 +136,27 @@ def test_config5_whole_tensor_doubling_property():
         assert torch.equal(b[name], a[name] * 2), name
 
 
+def test_config4_whole_tensor_properties():
+    """Size-independent checks at configuration 4 over whole tensors.  Doubling dO is exact in bf16 and in
+    every fp32 sum, so all five gradients double bit for bit while out and lse stay; heads are
+    independent, so permuting the heads of every input permutes every result bit for bit (each
+    (batch, head) lands on other workgroups and another XCD)."""
+    inp = make_inputs(1, 8192, 16, 128, seed=3, dtype=torch.bfloat16)
+    a = run_device(inp, 512, 32, flags=MFMA)
+    inp2 = list(inp)
+    inp2[5] = inp[5] * 2
+    b = run_device(inp2, 512, 32, flags=MFMA)
+    assert torch.equal(b["out"], a["out"]) and torch.equal(b["lse"], a["lse"])
+    for name in GRADS:
+        assert torch.isfinite(a[name].float()).all(), name
+        assert torch.equal(b[name], a[name] * 2), name
+    perm = torch.randperm(16, generator=torch.Generator().manual_seed(5))
+    c = run_device([t[:, :, perm].contiguous() for t in inp], 512, 32, flags=MFMA)
+    assert torch.equal(c["lse"], a["lse"][:, perm])
+    for name in ("out",) + tuple(GRADS):
+        assert torch.equal(c[name], a[name][:, :, perm]), name
+
+
 def test_needs_input_grad_subsets_and_determinism():
     from simplical_attn_amd import TwoSimplicialAttentionFunction as Fn
     dev = torch.device("cuda:0")
