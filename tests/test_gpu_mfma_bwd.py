@@ -31,6 +31,9 @@ SMALL = [  # B, N, H, D, w1, w2, k2_bias, v2_bias
     (1, 200, 1, 32, 64, 32, 0.0, 0.0),
     (1, 200, 1, 128, 16, 150, 0.0, 0.1),     # K' window too wide for the on-chip kernels: workspace kernels
     (1, 180, 2, 128, 40, 100, 0.2, 0.0),     # K'-side on chip (q, dO rows from global memory), K-side workspace kernel
+    (1, 150, 1, 128, 20, 65, 0.0, 0.0),      # first K' window beyond the K-side on-chip kernel (64 is its last)
+    (1, 190, 1, 128, 12, 113, 0.0, 0.0),     # last K' window of the K'-side on-chip kernel
+    (1, 190, 1, 128, 12, 114, 0.0, 0.0),     # first one beyond it
 ]
 
 
