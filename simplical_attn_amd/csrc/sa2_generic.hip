@@ -363,6 +363,37 @@ __global__ __launch_bounds__(256) void rowdot_kernel(Tensor out, Tensor dout, fl
     if (lane == 0) dsum[row] = s;
 }
 
+// The same for 16-bit elements with 16-byte aligned rows and D = 8 << n: a lane takes eight
+// consecutive elements of a row in one 16-byte load per tensor, D / 8 lanes share a row, a
+// wavefront covers 512 / D rows.
+template <typename T>
+__global__ __launch_bounds__(256) void rowdot_vec_kernel(Tensor out, Tensor dout, float* dsum, int N, int H, int lpr_log2,
+                                                         int64_t rows) {
+    const int lane = threadIdx.x & 63;
+    const int lpr = 1 << lpr_log2;                        // lanes per row
+    const int64_t row = (((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) << (6 - lpr_log2)) + (lane >> lpr_log2);
+    const int sub = lane & (lpr - 1);
+    float s = 0.f;
+    if (row < rows) {
+        const int i = (int)(row % N);
+        const int bh = (int)(row / N);
+        const int b = bh / H, h = bh - b * H;
+        const uint4 o = *(const uint4*)((const T*)out.p + out.off(b, i, h) + sub * 8);
+        const uint4 g = *(const uint4*)((const T*)dout.p + dout.off(b, i, h) + sub * 8);
+        const uint32_t ow[4] = {o.x, o.y, o.z, o.w}, gw[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            union { uint32_t u; T h[2]; } a, c;
+            a.u = ow[t];
+            c.u = gw[t];
+            s = fmaf(to_float(a.h[0]), to_float(c.h[0]), s);
+            s = fmaf(to_float(a.h[1]), to_float(c.h[1]), s);
+        }
+    }
+    for (int off = lpr >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (row < rows && sub == 0) dsum[row] = s;
+}
+
 template <typename F>
 int dispatch_dtype(int dtype, F&& f) {
     switch (dtype) {
@@ -387,8 +418,25 @@ int launch_rowdot(const Tensor& out, const Tensor& dout, float* dsum, int B, int
     const int64_t rows = (int64_t)B * H * N;
     const int64_t blocks = (rows + 3) / 4;
     if (blocks > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
+    // 16-bit elements, D = 8, 16, .. 256 and 16-byte aligned rows: the vector kernel
+    auto aligned = [&](const Tensor& t) {
+        return ((uintptr_t)t.p & 15u) == 0 && (B == 1 || t.sb % 8 == 0) && (N == 1 || t.sn % 8 == 0) && (H == 1 || t.sh % 8 == 0);
+    };
+    int lpr_log2 = -1;
+    for (int n = 0; n <= 5; ++n)
+        if (D == (8 << n)) lpr_log2 = n;
+    const bool vec = dtype != SA2_F32 && lpr_log2 >= 0 && aligned(out) && aligned(dout);
     return dispatch_dtype(dtype, [&](auto* tag) {
         using T = std::remove_pointer_t<decltype(tag)>;
+        if constexpr (sizeof(T) == 2) {
+            if (vec) {
+                const int64_t per_block = (int64_t)4 << (6 - lpr_log2);           // rows per workgroup
+                const int64_t vblocks = (rows + per_block - 1) / per_block;
+                hipLaunchKernelGGL(rowdot_vec_kernel<T>, dim3((unsigned)vblocks), dim3(256), 0, st, out, dout, dsum, N, H,
+                                   lpr_log2, rows);
+                return check_launch();
+            }
+        }
         hipLaunchKernelGGL(rowdot_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, st, out, dout, dsum, N, H, D, rows);
         return check_launch();
     });

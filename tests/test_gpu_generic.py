@@ -231,6 +231,24 @@ def test_rowdot():
     assert torch.equal(got, want.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("D", [16, 32, 64, 128, 256, 40])
+def test_rowdot_kernels(D, dtype):
+    """The 16-byte-per-lane kernel (16-bit elements, D = 8 << n, aligned rows), the element-wise one
+    (everything else), and views whose rows are not 16-byte aligned."""
+    from simplical_attn_amd import simplicial_rowdot
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(D)
+    a = torch.randn(2, 37, 3, D, generator=g).to(dtype).to(dev)
+    b = torch.randn(2, 37, 3, D, generator=g).to(dtype).to(dev)
+    want = (a.double() * b.double()).sum(-1).permute(0, 2, 1)
+    assert torch.allclose(simplicial_rowdot(a, b).double(), want, rtol=1e-5, atol=1e-4)
+    wide = torch.randn(2, 37, 3, D + 4, generator=g).to(dtype).to(dev)        # rows 8 bytes off the 16-byte grid
+    av = wide[..., 4:]
+    want = (av.double() * b.double()).sum(-1).permute(0, 2, 1)
+    assert torch.allclose(simplicial_rowdot(av, b).double(), want, rtol=1e-5, atol=1e-4)
+
+
 def test_broadcast_views_are_accepted():
     """Losses that hand backward an expanded gradient (stride 0 along a summed axis) and keys
     expanded over heads (stride 0 on H) run, as the reference's stride-generic launch lets them
