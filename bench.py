@@ -11,9 +11,11 @@ w1=512 w2=32.  Prints ONE JSON line:
   metric/value   forward+backward algorithmic TFLOP/s: 16*D*T flops per step,
                  T = number of valid (i,j,k) triples (matmul flops only, 2 per
                  MAC: 4*D*T forward, 12*D*T backward)
-  roofline       the single kernel that dominates the step, against the bf16 dense
-                 MFMA peak (achieved = that kernel's algorithmic flops / its duration,
-                 measured here with events on the launch stream); `mfma_busy` and
+  roofline       the kernel group that takes the longest in the step (whichever of the
+                 forward, the K-side and the K'-side backward measures longest in this
+                 run), against the bf16 dense MFMA peak (achieved = that group's
+                 algorithmic flops / its duration, measured here with events on the
+                 launch stream); `groups` lists all three; `mfma_busy` and
                  `traffic` are rocprofv3 counter results read from profiles/
                  (measured in separate profiler runs of this same script)
   kernels        the same for every kernel group of the step, plus HBM GB/s
@@ -387,13 +389,14 @@ def main():
     for name in ("backward_k_side", "backward_kprime_side", "backward"):
         kernels[name]["frac_at_observed_clock"] = kernels[name]["tflops"] / peak_at(clocks["backward"])
 
-    # The dominant kernel: the K-side kernel is one launch, so its own duration is measured here
-    # (call with only dK, dV requested minus the row-dot kernel); the other two groups hold three
-    # launches each (their pre-pass and a short epilogue kernel beside the main one).
-    dominant = "backward_k_side"
-    longest_group = max(("forward", "backward_k_side", "backward_kprime_side"), key=lambda k: kernels[k]["ms"])
+    # The dominant kernel group: the one that takes the longest in the step.  The K-side kernel is a
+    # single launch (its duration here: the call that requests only dK and dV, minus the row-dot
+    # kernel); the forward and the K'-side group hold three launches each (a pre-pass and a short
+    # epilogue kernel beside the main one), of which the main kernel is more than nine tenths.
+    dominant = max(("forward", "backward_k_side", "backward_kprime_side"), key=lambda k: kernels[k]["ms"])
     roofline = {
-        "bound": "mfma", "kernel": kernels[dominant]["kernel"],
+        "bound": "mfma", "kernel": kernels[dominant]["kernel"], "group": dominant,
+        "launches": kernels[dominant]["launches"],
         "achieved": kernels[dominant]["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
         "frac": kernels[dominant]["frac_bf16_peak"],
         "traffic": kernels[dominant]["traffic"],
@@ -402,8 +405,8 @@ def main():
         "mfma_busy": kernels[dominant]["mfma_busy"],
         "frac_at_observed_clock": kernels[dominant]["frac_at_observed_clock"],
         "counters_from": key_sources.get(wl),
-        "longest_group": {"name": longest_group, "kernel": kernels[longest_group]["kernel"],
-                          "ms": kernels[longest_group]["ms"], "frac": kernels[longest_group]["frac_bf16_peak"]},
+        "groups": {k: {"ms": kernels[k]["ms"], "frac": kernels[k]["frac_bf16_peak"]}
+                   for k in ("forward", "backward_k_side", "backward_kprime_side")},
     }
     roofline_fwd = {
         "bound": "mfma", "kernel": kernels["forward"]["kernel"], "achieved": kernels["forward"]["tflops"],

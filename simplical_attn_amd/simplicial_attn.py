@@ -17,9 +17,11 @@ from . import _lib
 
 _DTYPES = {torch.float32: _lib.SA2_F32, torch.bfloat16: _lib.SA2_BF16, torch.float16: _lib.SA2_F16}
 
-# Window convention: True = closed windows [i-w, i] as the reference's PyTorch
-# oracle defines them (simplicial/reference.py:41-45); False = half-open
-# (i-w, i] as the reference's device kernels mask (simplicial/kernels.py:133-136).
+# Window convention, an argument of every entry point below (``window_inclusive``):
+# True = closed windows [i-w, i] as the reference's PyTorch oracle defines them
+# (simplicial/reference.py:41-45); False = half-open (i-w, i] as the reference's device
+# kernels mask (simplicial/kernels.py:133-136).  This is only the default of that argument;
+# nothing reads it at call time.
 WINDOW_INCLUSIVE = True
 
 
@@ -28,11 +30,25 @@ def _check_inputs(q, k1, k2, v1, v2):
         raise ValueError("expected [batch, seq_len, num_heads, head_dim] tensors, got shape %s" % (tuple(q.shape),))
     if q.dtype not in _DTYPES:
         raise TypeError("unsupported dtype %s (float32, bfloat16, float16)" % q.dtype)
-    if not q.is_cuda:
-        raise RuntimeError("TwoSimplicialAttention runs on the GPU only; got a %s tensor" % q.device)
     for name, t in (("k1", k1), ("k2", k2), ("v1", v1), ("v2", v2)):
         if t.shape != q.shape or t.dtype != q.dtype or t.device != q.device:
             raise ValueError("%s must match q in shape, dtype and device" % name)
+    if not q.is_cuda:
+        raise RuntimeError("TwoSimplicialAttention runs on the GPU only; got a %s tensor" % q.device)
+
+
+def _check_saved(q, out, lse, dout):
+    """The tensors a backward call gets beside the five inputs: their addresses go to the kernels
+    as they are, so everything the kernels assume is checked here."""
+    B, N, H, _ = q.shape
+    for name, t in (("out", out), ("dout", dout)):
+        if not isinstance(t, torch.Tensor) or t.shape != q.shape or t.dtype != q.dtype or t.device != q.device:
+            raise ValueError("%s must match q in shape, dtype and device" % name)
+    if not isinstance(lse, torch.Tensor) or lse.dtype != torch.float32 or lse.device != q.device:
+        raise ValueError("lse must be a float32 tensor on q's device")
+    if tuple(lse.shape) != (B, H, N) or not lse.is_contiguous():
+        raise ValueError("lse must be contiguous [batch, num_heads, seq_len] = %s, got shape %s strides %s"
+                         % ((B, H, N), tuple(lse.shape), lse.stride()))
 
 
 def _rows(t):
@@ -66,7 +82,7 @@ def _stream(t):
 
 
 def simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0, flags=_lib.FLAG_AUTO,
-                       window_inclusive=None):
+                       window_inclusive=True):
     """Runs the forward kernel; returns (output like q, LSE [B,H,N] fp32).
     Replaces the launch in triton_impl.py:23-51."""
     _check_inputs(q, k1, k2, v1, v2)
@@ -74,8 +90,6 @@ def simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bi
     B, N, H, D = q.shape
     if scale is None:
         scale = 1.0 / math.sqrt(D)
-    if window_inclusive is None:
-        window_inclusive = WINDOW_INCLUSIVE
     width = _pad_head_dim(D, q.dtype, flags)
     if width != D:
         out, lse = simplicial_forward(*(_padded(t, width) for t in (q, k1, k2, v1, v2)), w1, w2, scale, k2_bias,
@@ -94,15 +108,18 @@ def simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bi
 
 
 def simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0,
-                        needs=(True, True, True, True, True), flags=_lib.FLAG_AUTO, window_inclusive=None):
+                        needs=(True, True, True, True, True), flags=_lib.FLAG_AUTO, window_inclusive=True):
     """Runs the backward kernels; returns (dq, dk1, dk2, dv1, dv2) in the input
-    dtype, None where ``needs`` is False.  Replaces triton_impl.py:61-158."""
+    dtype, None where ``needs`` is False.  Replaces triton_impl.py:61-158.
+    ``out`` and ``lse`` are what simplicial_forward returned for the same inputs and arguments."""
+    _check_inputs(q, k1, k2, v1, v2)
+    _check_saved(q, out, lse, dout)
+    if len(needs) != 5:
+        raise ValueError("needs must have five entries (dq, dk1, dk2, dv1, dv2), got %d" % len(needs))
     lib = _lib.load()
     B, N, H, D = q.shape
     if scale is None:
         scale = 1.0 / math.sqrt(D)
-    if window_inclusive is None:
-        window_inclusive = WINDOW_INCLUSIVE
     width = _pad_head_dim(D, q.dtype, flags)
     if width != D:
         grads = simplicial_backward(*(_padded(t, width) for t in (q, k1, k2, v1, v2, out)), lse, _padded(dout, width),
@@ -153,20 +170,27 @@ class TwoSimplicialAttentionFunction(torch.autograd.Function):
     """autograd Function with the reference's argument list
     (simplicial/triton_impl.py:19): forward saves (q, k1, k2, v1, v2, output,
     LSE) as triton_impl.py:54 does; backward returns five gradients in the
-    inputs' dtype and five None (triton_impl.py:157-158)."""
+    inputs' dtype and None for every other argument (triton_impl.py:157-158).
 
-    kernel_flags = _lib.FLAG_AUTO
+    Two trailing arguments beyond the reference's ten, both optional so that the reference's
+    positional call works unchanged: ``window_inclusive`` (True: closed windows [i-w, i] of
+    simplicial/reference.py:41-45; False: the half-open (i-w, i] of the reference's device
+    kernels, simplicial/kernels.py:133-136) and ``kernel_flags`` (kernel choice of the C ABI:
+    0 automatic, 1 fp32 FMA kernels, 2 MFMA kernels or an error).  Both travel in ``ctx``;
+    no process-wide state is read."""
 
     @staticmethod
-    def forward(ctx, q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias):
+    def forward(ctx, q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias, window_inclusive=True,
+                kernel_flags=_lib.FLAG_AUTO):
         if scale is None:
             scale = 1.0 / math.sqrt(q.shape[-1])
-        flags = TwoSimplicialAttentionFunction.kernel_flags
-        out, lse = simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias, flags)
+        window_inclusive = bool(window_inclusive)
+        out, lse = simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias, kernel_flags,
+                                      window_inclusive)
         ctx.save_for_backward(q, k1, k2, v1, v2, out, lse)
         ctx.w1, ctx.w2, ctx.scale, ctx.k2_bias, ctx.v2_bias = w1, w2, scale, k2_bias, v2_bias
-        ctx.flags = flags
-        ctx.window_inclusive = WINDOW_INCLUSIVE
+        ctx.flags = kernel_flags
+        ctx.window_inclusive = window_inclusive
         return out
 
     @staticmethod
@@ -175,47 +199,26 @@ class TwoSimplicialAttentionFunction(torch.autograd.Function):
         grads = simplicial_backward(q, k1, k2, v1, v2, out, lse, grad_output, ctx.w1, ctx.w2, ctx.scale,
                                     ctx.k2_bias, ctx.v2_bias, needs=tuple(ctx.needs_input_grad[:5]),
                                     flags=ctx.flags, window_inclusive=ctx.window_inclusive)
-        return (*grads, None, None, None, None, None)
+        # (autograd drops the trailing None entries of a call that left the optional arguments out)
+        return (*grads, None, None, None, None, None, None, None)
 
 
-class _ExactFunction(torch.autograd.Function):
-    """The same operator on the fp32 FMA kernels (every product and sum in fp32, whatever the
-    element type of the tensors): the slow, exact path that plays the part of the reference's
-    PyTorch loop when results of the MFMA kernels are to be checked on the device."""
-
-    @staticmethod
-    def forward(ctx, q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias):
-        if scale is None:
-            scale = 1.0 / math.sqrt(q.shape[-1])
-        out, lse = simplicial_forward(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias, _lib.FLAG_FORCE_GENERIC)
-        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse)
-        ctx.w1, ctx.w2, ctx.scale, ctx.k2_bias, ctx.v2_bias = w1, w2, scale, k2_bias, v2_bias
-        ctx.window_inclusive = WINDOW_INCLUSIVE
-        return out
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        q, k1, k2, v1, v2, out, lse = ctx.saved_tensors
-        grads = simplicial_backward(q, k1, k2, v1, v2, out, lse, grad_output, ctx.w1, ctx.w2, ctx.scale,
-                                    ctx.k2_bias, ctx.v2_bias, needs=tuple(ctx.needs_input_grad[:5]),
-                                    flags=_lib.FLAG_FORCE_GENERIC, window_inclusive=ctx.window_inclusive)
-        return (*grads, None, None, None, None, None)
-
-
-def two_simplicial_attention_exact(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0):
+def two_simplicial_attention_exact(q, k1, k2, v1, v2, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0,
+                                   window_inclusive=True):
     """Argument list of the reference's PyTorch implementation (simplicial/reference.py:8-9), run
     on the fp32 FMA kernels on the GPU (same windows, bias and epsilon as reference.py:27-76),
     differentiable.  It is a device-side yardstick for the MFMA kernels: HIP kernels of this same
     library, NOT an independent reference and not a CPU path.  Comparing the operator with it is a
     kernel-against-kernel check."""
-    return _ExactFunction.apply(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias)
+    return TwoSimplicialAttentionFunction.apply(q, k1, k2, v1, v2, w1, w2, scale, k2_bias, v2_bias,
+                                                window_inclusive, _lib.FLAG_FORCE_GENERIC)
 
 
 class TwoSimplicialAttentionExact(torch.nn.Module):
     """Module wrapper of two_simplicial_attention_exact with the constructor of the reference's
     TwoSimplicialAttentionReference (simplicial/reference.py:79-103)."""
 
-    def __init__(self, head_dim, w1=64, w2=64, scale=None, k2_bias=0.0, v2_bias=0.0):
+    def __init__(self, head_dim, w1=64, w2=64, scale=None, k2_bias=0.0, v2_bias=0.0, *, window_inclusive=True):
         super().__init__()
         self.head_dim = head_dim
         self.w1 = w1
@@ -223,17 +226,20 @@ class TwoSimplicialAttentionExact(torch.nn.Module):
         self.scale = scale if scale is not None else (1.0 / math.sqrt(head_dim))
         self.k2_bias = k2_bias
         self.v2_bias = v2_bias
+        self.window_inclusive = bool(window_inclusive)
 
     def forward(self, q, k1, k2, v1, v2):
         return two_simplicial_attention_exact(q, k1, k2, v1, v2, self.w1, self.w2, self.scale,
-                                              self.k2_bias, self.v2_bias)
+                                              self.k2_bias, self.v2_bias, self.window_inclusive)
 
 
 class TwoSimplicialAttention(torch.nn.Module):
     """Module wrapper with the reference's constructor and call signature
-    (simplicial/triton_impl.py:161-186); holds no parameters."""
+    (simplicial/triton_impl.py:161-186); holds no parameters.  The keyword-only
+    ``window_inclusive=False`` selects the half-open windows (i-w, i] of the reference's device
+    kernels (simplicial/kernels.py:133-136) for callers that migrate from them."""
 
-    def __init__(self, head_dim, w1=64, w2=64, scale=None, k2_bias=0.0, v2_bias=0.0):
+    def __init__(self, head_dim, w1=64, w2=64, scale=None, k2_bias=0.0, v2_bias=0.0, *, window_inclusive=True):
         super().__init__()
         self.head_dim = head_dim
         self.w1 = w1
@@ -241,7 +247,8 @@ class TwoSimplicialAttention(torch.nn.Module):
         self.scale = scale if scale is not None else (1.0 / math.sqrt(head_dim))
         self.k2_bias = k2_bias
         self.v2_bias = v2_bias
+        self.window_inclusive = bool(window_inclusive)
 
     def forward(self, q, k1, k2, v1, v2):
         return TwoSimplicialAttentionFunction.apply(q, k1, k2, v1, v2, self.w1, self.w2, self.scale,
-                                                    self.k2_bias, self.v2_bias)
+                                                    self.k2_bias, self.v2_bias, self.window_inclusive)

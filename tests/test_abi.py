@@ -73,14 +73,76 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F32) == 0
 
 
+def test_forced_mfma_refuses_layouts_its_loads_cannot_take(lib):
+    """The MFMA kernels move 16-byte chunks with 32-bit row offsets.  A 16-bit tensor whose rows are
+    off the 16-byte grid, whose rows span 2^31 elements or more, an unsupported head_dim or fp32 must
+    never reach them: with SA2_FLAG_FORCE_MFMA the call returns SA2_ERR_UNSUPPORTED and launches
+    nothing (pointers here are never dereferenced; with SA2_FLAG_AUTO the same problems take the
+    fp32 kernels, which the GPU tests cover)."""
+    B, N, H, D = 1, 64, 2, 128
+    good = (N * H * D, H * D, D)
+    base = 1 << 20                                     # 16-byte aligned, never dereferenced
+    FORCE, UNSUPPORTED = _lib.FLAG_FORCE_MFMA, -8
+
+    def fwd(ptrs=None, strides=None, N=N, D=D, dtype=_lib.SA2_BF16):
+        ptrs = ptrs or [base] * 6
+        st = _lib.stride_array(strides or [good] * 6)
+        return lib.sa2_forward(*[ctypes.c_void_p(x) for x in ptrs], ctypes.c_void_p(base), B, N, H, D, st,
+                               16, 8, 0.1, 0.0, 0.0, dtype, 1, FORCE, None)
+
+    def bwd(ptrs=None, strides=None, dtype=_lib.SA2_BF16):
+        ptrs = ptrs or [base] * 12                     # q k1 k2 v1 v2 out dout dq dk1 dk2 dv1 dv2
+        st = _lib.stride_array(strides or [good] * 12)
+        ws = lib.sa2_bwd_workspace_bytes(B, N, H, D, 16, 8, dtype, FORCE)
+        args = [ctypes.c_void_p(x) for x in ptrs[:7]] + [ctypes.c_void_p(base)] + [ctypes.c_void_p(x) for x in ptrs[7:]]
+        return lib.sa2_backward(*args, ctypes.c_void_p(base), ws, B, N, H, D, st, 16, 8, 0.1, 0.0, 0.0, dtype, 1,
+                                FORCE, None)
+
+    for t in range(6):                                 # a base pointer 8 bytes off the grid, tensor by tensor
+        ptrs = [base] * 6
+        ptrs[t] = base + 8
+        assert fwd(ptrs=ptrs) == UNSUPPORTED, t
+    for axis in (1, 2):                                # a sequence or head stride that is not a multiple of 8 elements
+        st = [good] * 6                                # (the batch axis has size 1 here and may carry any stride)
+        odd = list(good)
+        odd[axis] += 4
+        st[1] = tuple(odd)
+        assert fwd(strides=st) == UNSUPPORTED, axis
+    st = [good] * 6
+    st[3] = (good[0], (1 << 31) // (N - 1) // 8 * 8 + 8, D)      # (N-1) * stride_n reaches 2^31 elements
+    assert fwd(strides=st) == UNSUPPORTED
+    st[3] = (good[0], 1 << 40, D)
+    assert fwd(strides=st) == UNSUPPORTED
+    assert fwd(D=48, strides=[(N * H * 48, H * 48, 48)] * 6) == UNSUPPORTED
+    assert fwd(dtype=_lib.SA2_F32) == UNSUPPORTED
+    # backward: the same guards, and they cover dout and the gradient tensors too
+    for t in range(12):
+        ptrs = [base] * 12
+        ptrs[t] = base + 8
+        assert bwd(ptrs=ptrs) == UNSUPPORTED, t
+    st = [good] * 12
+    st[6] = (good[0], H * D + 4, D)
+    assert bwd(strides=st) == UNSUPPORTED
+    assert bwd(dtype=_lib.SA2_F32) == UNSUPPORTED
+
+
 def test_operator_interface_matches_reference():
     """Names, argument order and defaults of simplicial/triton_impl.py:19, 61, 164, 173."""
     import simplical_attn_amd as sa
     sig = inspect.signature(sa.TwoSimplicialAttention.__init__)
-    assert list(sig.parameters) == ["self", "head_dim", "w1", "w2", "scale", "k2_bias", "v2_bias"]
+    positional = [k for k, v in sig.parameters.items() if v.kind == v.POSITIONAL_OR_KEYWORD]
+    assert positional == ["self", "head_dim", "w1", "w2", "scale", "k2_bias", "v2_bias"]
     assert [sig.parameters[k].default for k in ("w1", "w2", "scale", "k2_bias", "v2_bias")] == [64, 64, None, 0.0, 0.0]
+    # what this build adds is keyword-only and defaults to the reference's behaviour
+    extra = {k: v for k, v in sig.parameters.items() if v.kind == v.KEYWORD_ONLY}
+    assert list(extra) == ["window_inclusive"] and extra["window_inclusive"].default is True
     fsig = inspect.signature(sa.TwoSimplicialAttentionFunction.forward)
-    assert list(fsig.parameters) == ["ctx", "q", "k1", "k2", "v1", "v2", "w1", "w2", "scale", "k2_bias", "v2_bias"]
+    names = list(fsig.parameters)
+    assert names[:11] == ["ctx", "q", "k1", "k2", "v1", "v2", "w1", "w2", "scale", "k2_bias", "v2_bias"]
+    # the reference's ten-argument positional call still works: everything after it is defaulted
+    assert names[11:] == ["window_inclusive", "kernel_flags"]
+    assert fsig.parameters["window_inclusive"].default is True and fsig.parameters["kernel_flags"].default == 0
+    assert not hasattr(sa.TwoSimplicialAttentionFunction, "kernel_flags")      # no process-wide switches
     m = sa.TwoSimplicialAttention(64)
     assert m.scale == 1.0 / 8.0 and m.w1 == 64 and m.w2 == 64 and len(list(m.parameters())) == 0
     assert list(inspect.signature(m.forward).parameters) == ["q", "k1", "k2", "v1", "v2"]
@@ -91,7 +153,7 @@ def test_reference_package_names():
     reference's signature or raises an AttributeError that says what to use instead."""
     import simplical_attn_amd as sa
     rsig = inspect.signature(sa.two_simplicial_attention_exact)
-    assert list(rsig.parameters) == ["q", "k1", "k2", "v1", "v2", "w1", "w2", "scale", "k2_bias", "v2_bias"]
+    assert list(rsig.parameters)[:10] == ["q", "k1", "k2", "v1", "v2", "w1", "w2", "scale", "k2_bias", "v2_bias"]
     assert [rsig.parameters[k].default for k in ("scale", "k2_bias", "v2_bias")] == [None, 0.0, 0.0]
     m = sa.TwoSimplicialAttentionExact(16, 4, 4)
     assert m.scale == 0.25 and list(inspect.signature(m.forward).parameters) == ["q", "k1", "k2", "v1", "v2"]
@@ -109,6 +171,39 @@ def test_reference_package_names():
     x = torch.zeros(1, 8, 1, 16)
     with pytest.raises(RuntimeError, match="GPU only"):
         sa.two_simplicial_attention_exact(x, x, x, x, x, 4, 4)
+
+
+def test_backward_validates_saved_tensors_before_any_pointer_is_taken():
+    """simplicial_backward is reachable by any caller (and through the torch.library op): out, dout
+    and lse are checked against q before their addresses go to the kernels.  The input checks run
+    first, so these tensors can live on the CPU here: a CPU q fails with the 'GPU only' error, and
+    everything checked before that fails with a ValueError."""
+    import simplical_attn_amd as sa
+    from simplical_attn_amd import simplicial_attn as host
+    B, N, H, D = 1, 8, 2, 16
+    x = torch.zeros(B, N, H, D)
+    lse = torch.zeros(B, H, N)
+    # the checks themselves, on tensors of one device
+    host._check_saved(x, x, lse, x)
+    for bad_out in (x[:, :4], x.double(), x[0]):
+        with pytest.raises(ValueError, match="out must match q"):
+            host._check_saved(x, bad_out, lse, x)
+    for bad_dout in (torch.zeros(B, N, H, D + 1), x.half()):
+        with pytest.raises(ValueError, match="dout must match q"):
+            host._check_saved(x, x, lse, bad_dout)
+    with pytest.raises(ValueError, match="float32"):
+        host._check_saved(x, x, lse.double(), x)
+    with pytest.raises(ValueError, match="contiguous"):
+        host._check_saved(x, x, torch.zeros(B, N, H), x)                    # the reference helper's [B,N,H] order
+    with pytest.raises(ValueError, match="contiguous"):
+        host._check_saved(x, x, torch.zeros(B, N, H).transpose(1, 2), x)    # right shape, wrong strides
+    with pytest.raises(ValueError, match="lse must be"):
+        host._check_saved(x, x, None, x)
+    # and the entry point runs them (after the input checks, which refuse CPU tensors)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sa.simplicial_backward(x, x, x, x, x, x, lse, x, 4, 4)
+    with pytest.raises(ValueError, match="k1 must match q"):
+        sa.simplicial_backward(x, x[:, :4], x, x, x, x, lse, x, 4, 4)
 
 
 def test_cpu_tensors_fail_loudly():

@@ -168,19 +168,15 @@ def test_needs_input_grad_subsets_and_determinism():
     again = run_device(inp, 60, 12, flags=MFMA)
     for name in GRADS:
         assert torch.equal(full[name], again[name]), name
-    old = Fn.kernel_flags
-    Fn.kernel_flags = MFMA            # the same kernel choice as `full` (pre-pass kernels included)
-    try:
-        for subset in ((0,), (1, 3), (2, 4), (0, 1, 2)):
-            leaves = [x.to(dev).requires_grad_(t in subset) for t, x in enumerate(inp[:5])]
-            Fn.apply(*leaves, 60, 12, None, 0.0, 0.0).backward(inp[5].to(dev))
-            for t, name in enumerate(GRADS):
-                if t in subset:
-                    assert torch.equal(leaves[t].grad, full[name]), name
-                else:
-                    assert leaves[t].grad is None
-    finally:
-        Fn.kernel_flags = old
+    for subset in ((0,), (1, 3), (2, 4), (0, 1, 2)):
+        leaves = [x.to(dev).requires_grad_(t in subset) for t, x in enumerate(inp[:5])]
+        # the same kernel choice as `full` (pre-pass kernels included)
+        Fn.apply(*leaves, 60, 12, None, 0.0, 0.0, True, MFMA).backward(inp[5].to(dev))
+        for t, name in enumerate(GRADS):
+            if t in subset:
+                assert torch.equal(leaves[t].grad, full[name]), name
+            else:
+                assert leaves[t].grad is None
 
 
 def test_headline_shape_scaling_and_swap_properties():

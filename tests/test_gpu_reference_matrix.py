@@ -9,6 +9,18 @@ from oracle import simplicial_oracle as orc
 
 pytestmark = pytest.mark.gpu
 TOL = {torch.float16: 1e-2, torch.bfloat16: 1e-2, torch.float32: 1e-4}     # atol = rtol (test_correctness.py:45-49)
+# The reference's inputs are scaled by 0.1, so its outputs are ~1e-3 and its absolute bars pass for almost
+# any output.  Beside them every comparison here also holds max|diff| to a fraction of max|ref|: the
+# 16-bit parity bars, and 1e-5 for fp32 (the fp32 contract of this build).
+REL = {torch.float16: 1e-2, torch.bfloat16: 2e-2, torch.float32: 1e-5}
+
+
+def _close(out, want, dtype):
+    """The reference's own allclose bar and, beside it, the relative one."""
+    got, ref = out.cpu().float(), want.float()
+    assert torch.allclose(got, ref, atol=TOL[dtype], rtol=TOL[dtype])
+    diff, scale = (got - ref).abs().max().item(), ref.abs().max().item()
+    assert diff <= REL[dtype] * scale, "max|diff| %.3e > %.1e * max|ref| %.3e" % (diff, REL[dtype], scale)
 
 
 def _inputs(B, N, H, D, dtype, seed, std=0.1):
@@ -35,8 +47,7 @@ def test_forward_vs_reference(shape, dtype):
     inp = _inputs(B, N, H, D, dtype, seed=N + D)
     out = _module(D, 16, 16)(*[x.cuda() for x in inp])
     assert out.dtype == dtype and out.shape == (B, N, H, D)
-    want = _oracle(inp, 16, 16).to(dtype)
-    assert torch.allclose(out.cpu().float(), want.float(), atol=TOL[dtype], rtol=TOL[dtype])
+    _close(out, _oracle(inp, 16, 16), dtype)
 
 
 @pytest.mark.parametrize("w", [(4, 4), (8, 8), (16, 16), (32, 32), (64, 64)])
@@ -44,8 +55,7 @@ def test_window_sizes(w):
     """test_correctness.py:179-198."""
     inp = _inputs(2, 128, 4, 64, torch.bfloat16, seed=5)
     out = _module(64, *w)(*[x.cuda() for x in inp])
-    want = _oracle(inp, *w).to(torch.bfloat16)
-    assert torch.allclose(out.cpu().float(), want.float(), atol=1e-2, rtol=1e-2)
+    _close(out, _oracle(inp, *w), torch.bfloat16)
 
 
 @pytest.mark.parametrize("bias", [(0.0, 0.0), (0.1, 0.2), (-0.1, -0.2), (1.0, 0.5)])
@@ -53,8 +63,7 @@ def test_bias_values(bias):
     """test_correctness.py:200-226."""
     inp = _inputs(2, 64, 2, 32, torch.bfloat16, seed=6)
     out = _module(32, 16, 16, k2_bias=bias[0], v2_bias=bias[1])(*[x.cuda() for x in inp])
-    want = _oracle(inp, 16, 16, *bias).to(torch.bfloat16)
-    assert torch.allclose(out.cpu().float(), want.float(), atol=1e-2, rtol=1e-2)
+    _close(out, _oracle(inp, 16, 16, *bias), torch.bfloat16)
 
 
 def test_backward_pass_basic_and_accumulation():

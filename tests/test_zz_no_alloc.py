@@ -13,27 +13,35 @@ pytestmark = pytest.mark.gpu
 DT = {torch.bfloat16: _lib.SA2_BF16, torch.float32: _lib.SA2_F32}
 
 
-def _both_backwards(shape, w, dtype, seed, flags):
+def _both_backwards(shape, w, dtype, seed, flags, inclusive=1, needs=(True,) * 5):
     import simplical_attn_amd as sa
     lib = _lib.load()
     dev = torch.device("cuda:0")
     B, N, H, D = shape
     q, k1, k2, v1, v2, dout = [t.to(dev) for t in make_inputs(B, N, H, D, seed, dtype)]
-    out, lse = sa.simplicial_forward(q, k1, k2, v1, v2, w[0], w[1], flags=flags)
+    out, lse = sa.simplicial_forward(q, k1, k2, v1, v2, w[0], w[1], flags=flags, window_inclusive=bool(inclusive))
     stream = torch.cuda.current_stream(dev).cuda_stream
     scale = D ** -0.5
     nbytes = lib.sa2_bwd_workspace_bytes(B, N, H, D, w[0], w[1], DT[dtype], flags)
     assert 0 < nbytes <= _lib.STATIC_WORKSPACE_BYTES
     results = []
+    free_before = None
     for static in (False, True):
         # gradients start from different garbage in the two runs: every element must be written
         grads = [torch.full_like(q, 7.0 if static else -3.0) for _ in range(5)]
         strides = _lib.stride_array([(t.stride(0), t.stride(1), t.stride(2))
                                      for t in (q, k1, k2, v1, v2, out, dout, *grads)])
-        head = [t.data_ptr() for t in (q, k1, k2, v1, v2, out, dout, lse, *grads)]
-        tail = [B, N, H, D, strides, w[0], w[1], scale, 0.0, 0.0, DT[dtype], 1, flags, stream]
+        head = [t.data_ptr() for t in (q, k1, k2, v1, v2, out, dout, lse)]
+        head += [g.data_ptr() if need else None for g, need in zip(grads, needs)]      # NULL = not needed
+        tail = [B, N, H, D, strides, w[0], w[1], scale, 0.0, 0.0, DT[dtype], inclusive, flags, stream]
         if static:
+            torch.cuda.synchronize()
+            free_before = torch.cuda.mem_get_info(dev)[0]
             _lib.check(lib.sa2_backward_static_workspace(*head, *tail))
+            torch.cuda.synchronize()
+            # the call allocates nothing: the device's free memory is what it was (nothing else runs
+            # between the two readings; torch's own allocator is not called either)
+            assert torch.cuda.mem_get_info(dev)[0] == free_before
         else:
             ws = torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=dev)
             _lib.check(lib.sa2_backward(*head, ws.data_ptr(), ws.numel(), *tail))
@@ -47,12 +55,28 @@ def _both_backwards(shape, w, dtype, seed, flags):
     (torch.bfloat16, _lib.FLAG_FORCE_MFMA, ((2, 512, 2, 64), (64, 32)), ((1, 96, 2, 64), (32, 5))),
     (torch.float32, _lib.FLAG_AUTO, ((1, 192, 2, 64), (32, 16)), ((1, 70, 1, 64), (16, 4))),
 ])
-def test_static_workspace_backward_matches_caller_workspace(dtype, flags, first, second):
+@pytest.mark.parametrize("inclusive", [1, 0])
+def test_static_workspace_backward_matches_caller_workspace(dtype, flags, first, second, inclusive):
     for call, (shape, w) in enumerate((first, second)):
-        plain, static = _both_backwards(shape, w, dtype, seed=11 + call, flags=flags)
+        plain, static = _both_backwards(shape, w, dtype, seed=11 + call, flags=flags, inclusive=inclusive)
         for name, a, b in zip(("dq", "dk1", "dk2", "dv1", "dv2"), plain, static):
             assert torch.isfinite(b.float()).all(), (call, name)
             assert torch.equal(a, b), "call %d, %s: static-workspace result differs" % (call, name)
+
+
+@pytest.mark.parametrize("needs", [(False, True, False, True, True), (True, False, True, False, False)])
+def test_static_workspace_backward_with_null_gradients(needs):
+    """NULL gradient pointers (needs_input_grad false): the requested gradients equal the caller-workspace
+    entry point's, the tensors behind the NULL pointers are never written (they are not even passed)."""
+    for dtype, flags, shape, w in ((torch.bfloat16, _lib.FLAG_FORCE_MFMA, (1, 320, 2, 128), (64, 16)),
+                                   (torch.float32, _lib.FLAG_AUTO, (1, 100, 2, 64), (24, 6))):
+        plain, static = _both_backwards(shape, w, dtype, seed=5, flags=flags, needs=needs)
+        full, _ = _both_backwards(shape, w, dtype, seed=5, flags=flags)
+        for name, need, a, b, f in zip(("dq", "dk1", "dk2", "dv1", "dv2"), needs, plain, static, full):
+            if need:
+                assert torch.equal(a, b) and torch.equal(b, f), name
+            else:
+                assert (b == 7.0).all() and (a == -3.0).all(), name          # the fill values: untouched
 
 
 def test_static_workspace_rejects_what_does_not_fit():

@@ -100,21 +100,15 @@ def run_device(inputs, w1, w2, scale=None, k2_bias=0.0, v2_bias=0.0, flags=0, ba
     """Runs the HIP path through the autograd Function on cuda:0; returns the
     same dict as oracle_all (tensors on the GPU) plus lse from a direct call."""
     import simplical_attn_amd as sa
-    from simplical_attn_amd import simplicial_attn as host
-    Fn = host.TwoSimplicialAttentionFunction
+    Fn = sa.TwoSimplicialAttentionFunction
     dev = torch.device("cuda:0")
     leaves = [x.to(dev).requires_grad_(backward) for x in inputs[:5]]
-    old = Fn.kernel_flags, host.WINDOW_INCLUSIVE
-    Fn.kernel_flags, host.WINDOW_INCLUSIVE = flags, inclusive
-    try:
-        out = Fn.apply(*leaves, w1, w2, scale, k2_bias, v2_bias)
-        res = {"out": out.detach()}
-        _, res["lse"] = sa.simplicial_forward(*[x.detach() for x in leaves], w1, w2, scale, k2_bias, v2_bias,
-                                              flags=flags, window_inclusive=inclusive)
-        if backward:
-            out.backward(inputs[5].to(dev))
-            for name, leaf in zip(("dq", "dk1", "dk2", "dv1", "dv2"), leaves):
-                res[name] = leaf.grad
-    finally:
-        Fn.kernel_flags, host.WINDOW_INCLUSIVE = old
+    out = Fn.apply(*leaves, w1, w2, scale, k2_bias, v2_bias, inclusive, flags)
+    res = {"out": out.detach()}
+    _, res["lse"] = sa.simplicial_forward(*[x.detach() for x in leaves], w1, w2, scale, k2_bias, v2_bias,
+                                          flags=flags, window_inclusive=inclusive)
+    if backward:
+        out.backward(inputs[5].to(dev))
+        for name, leaf in zip(("dq", "dk1", "dk2", "dv1", "dv2"), leaves):
+            res[name] = leaf.grad
     return res
