@@ -96,14 +96,25 @@ void* static_workspace() {
 
 size_t dsum_bytes(int B, int N, int H) { return align_up((size_t)B * H * N * sizeof(float), 256); }
 
-bool pick_mfma(const Problem& p, int dtype, unsigned flags, bool backward, int* status) {
+// Which kernels a call takes: the fp32 FMA kernels, the 16-bit MFMA kernels, or the fp32 MFMA kernels.
+enum KernelPath { PATH_GENERIC, PATH_MFMA16, PATH_MFMA32 };
+
+KernelPath pick_path(const Problem& p, int dtype, unsigned flags, bool backward, int* status) {
     *status = SA2_OK;
-    if (flags & SA2_FLAG_FORCE_GENERIC) return false;
-    const bool ok = (backward ? mfma_bwd_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)
-                              : mfma_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)) &&
-                    mfma_layout_ok(p, backward);
-    if (!ok && (flags & SA2_FLAG_FORCE_MFMA)) *status = SA2_ERR_UNSUPPORTED;
-    return ok;
+    if (flags & SA2_FLAG_FORCE_GENERIC) return PATH_GENERIC;
+    KernelPath path = PATH_GENERIC;
+    if (dtype == SA2_F32) {
+        const bool ok = (backward ? f32_mfma_bwd_supported(p.D, p.w2, dtype) : f32_mfma_supported(p.D, dtype)) &&
+                        f32_mfma_layout_ok(p, backward);
+        if (ok) path = PATH_MFMA32;
+    } else {
+        const bool ok = (backward ? mfma_bwd_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)
+                                  : mfma_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)) &&
+                        mfma_layout_ok(p, backward);
+        if (ok) path = PATH_MFMA16;
+    }
+    if (path == PATH_GENERIC && (flags & SA2_FLAG_FORCE_MFMA)) *status = SA2_ERR_UNSUPPORTED;
+    return path;
 }
 
 }  // namespace
@@ -132,7 +143,7 @@ const char* sa2_strerror(int status) {
 
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype) {
     if (check_dims(B, N, H, D, w1, w2, dtype, 1) != SA2_OK) return 0;
-    return mfma_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype) ? 1 : 0;
+    return (mfma_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype) || f32_mfma_supported(D, dtype)) ? 1 : 0;
 }
 
 int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
@@ -161,9 +172,10 @@ int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, c
     p.force_prepass = (flags & SA2_FLAG_FORCE_MFMA) ? 1 : 0;
 
     hipStream_t st = (hipStream_t)hip_stream;
-    const bool mfma = pick_mfma(p, dtype, flags, false, &rc);
+    const KernelPath path = pick_path(p, dtype, flags, false, &rc);
     if (rc != SA2_OK) return rc;
-    return mfma ? launch_mfma_fwd(p, dtype, st) : launch_generic_fwd(p, dtype, st);
+    return path == PATH_MFMA16 ? launch_mfma_fwd(p, dtype, st)
+           : path == PATH_MFMA32 ? launch_f32_mfma_fwd(p, st) : launch_generic_fwd(p, dtype, st);
 }
 
 size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int dtype, unsigned flags) {
@@ -171,6 +183,10 @@ size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int d
     size_t scratch = generic_bwd_scratch_bytes(B, N, H, D, w1, w2);
     if (!(flags & SA2_FLAG_FORCE_GENERIC) && mfma_bwd_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype)) {
         const size_t m = mfma_bwd_scratch_bytes(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N));
+        if (m > scratch) scratch = m;
+    }
+    if (!(flags & SA2_FLAG_FORCE_GENERIC) && f32_mfma_bwd_supported(D, reach(w2, 1, N), dtype)) {
+        const size_t m = f32_mfma_bwd_scratch_bytes(B, N, H, D, reach(w2, 1, N));
         if (m > scratch) scratch = m;
     }
     return dsum_bytes(B, N, H) + align_up(scratch, 256) + 256;
@@ -219,9 +235,10 @@ int sa2_backward(const void* q, const void* k1, const void* k2, const void* v1, 
     p.force_prepass = (flags & SA2_FLAG_FORCE_MFMA) ? 1 : 0;
 
     hipStream_t st = (hipStream_t)hip_stream;
-    const bool mfma = pick_mfma(p, dtype, flags, true, &rc);
+    const KernelPath path = pick_path(p, dtype, flags, true, &rc);
     if (rc != SA2_OK) return rc;
-    return mfma ? launch_mfma_bwd(p, dtype, st) : launch_generic_bwd(p, dtype, st);
+    return path == PATH_MFMA16 ? launch_mfma_bwd(p, dtype, st)
+           : path == PATH_MFMA32 ? launch_f32_mfma_bwd(p, st) : launch_generic_bwd(p, dtype, st);
 }
 
 int sa2_backward_static_workspace(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,

@@ -85,6 +85,13 @@ bool mfma_layout_ok(const Problem& p, bool backward);
 int launch_mfma_fwd(const Problem& p, int dtype, hipStream_t st);
 int launch_mfma_bwd(const Problem& p, int dtype, hipStream_t st);
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
+// fp32 tensors on the fp32 MFMA (head_dim 32, 64, 128; rows 16-byte aligned)
+bool f32_mfma_supported(int D, int dtype);
+bool f32_mfma_bwd_supported(int D, int w2, int dtype);
+bool f32_mfma_layout_ok(const Problem& p, bool backward);
+size_t f32_mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w2);
+int launch_f32_mfma_fwd(const Problem& p, hipStream_t st);
+int launch_f32_mfma_bwd(const Problem& p, hipStream_t st);
 // K'-side backward kernel (dQ, dK', dV') that keeps its partial sums on chip
 bool kp_fits(int D, int w2);
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2);

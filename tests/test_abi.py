@@ -70,7 +70,9 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.sa2_backward(one, one, one, one, one, one, one, one, one, one, one, one, one, one, 16,
                             1, 8, 2, 64, strides, 4, 4, 0.125, 0.0, 0.0, 0, 1, 0, None) == -6
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_BF16) == 1
-    assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F32) == 0
+    assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F32) == 1      # the fp32 MFMA kernels
+    assert lib.sa2_uses_mfma(1, 8192, 16, 256, 512, 32, _lib.SA2_F32) == 0
+    assert lib.sa2_uses_mfma(1, 8192, 16, 256, 512, 32, _lib.SA2_BF16) == 0
 
 
 def test_forced_mfma_refuses_layouts_its_loads_cannot_take(lib):
@@ -114,7 +116,13 @@ def test_forced_mfma_refuses_layouts_its_loads_cannot_take(lib):
     st[3] = (good[0], 1 << 40, D)
     assert fwd(strides=st) == UNSUPPORTED
     assert fwd(D=48, strides=[(N * H * 48, H * 48, 48)] * 6) == UNSUPPORTED
-    assert fwd(dtype=_lib.SA2_F32) == UNSUPPORTED
+    # fp32 has MFMA kernels of its own (head_dim 32, 64, 128; float4 loads: 16-byte aligned rows)
+    assert fwd(D=48, strides=[(N * H * 48, H * 48, 48)] * 6, dtype=_lib.SA2_F32) == UNSUPPORTED
+    assert fwd(D=256, strides=[(N * H * 256, H * 256, 256)] * 6, dtype=_lib.SA2_F32) == UNSUPPORTED
+    assert fwd(ptrs=[base, base, base + 8, base, base, base], dtype=_lib.SA2_F32) == UNSUPPORTED
+    st = [good] * 6
+    st[4] = (good[0], H * D + 2, D)
+    assert fwd(strides=st, dtype=_lib.SA2_F32) == UNSUPPORTED
     # backward: the same guards, and they cover dout and the gradient tensors too
     for t in range(12):
         ptrs = [base] * 12
@@ -123,7 +131,9 @@ def test_forced_mfma_refuses_layouts_its_loads_cannot_take(lib):
     st = [good] * 12
     st[6] = (good[0], H * D + 4, D)
     assert bwd(strides=st) == UNSUPPORTED
-    assert bwd(dtype=_lib.SA2_F32) == UNSUPPORTED
+    ptrs = [base] * 12
+    ptrs[9] = base + 4
+    assert bwd(ptrs=ptrs, dtype=_lib.SA2_F32) == UNSUPPORTED
 
 
 def test_operator_interface_matches_reference():
