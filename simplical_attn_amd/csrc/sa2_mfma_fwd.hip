@@ -22,9 +22,12 @@
 // LDS read of the step is complete by then), then the value MFMAs of tile t-1, which
 // only read registers and so run under the next step's tile request and operand reads.
 // A step is one basic block (mask and request are compile-time variants of it), so that
-// the compiler can place all of this between the MFMAs.  After each round of 8 units the wavefronts fold their
-// (m, l, R*v2) into the workgroup's fp32 accumulator through bf16 slabs in LDS,
-// each thread summing a fixed slice in a fixed order.
+// the compiler can place all of this between the MFMAs.  At head_dim 128, after each round of 8 units the
+// wavefronts fold their (m, l, R*v2) into the workgroup's fp32 accumulator through bf16 slabs in LDS,
+// each thread summing a fixed slice in a fixed order.  At head_dim 32 and 64 the registers allow a
+// second accumulator per wavefront: every wavefront keeps the running (m, l, sum of R*v2) of its own
+// units, rounds follow each other without a barrier of their own, and the eight are merged once at the
+// end through fp32 LDS in wavefront order.
 //
 // The logits are computed transposed (S^T = K1 . Q~^T) so that an expanded row
 // lives in one lane pair: exp2(S^T) is already laid out as the B operand of
@@ -53,6 +56,15 @@ struct Cfg {
     static constexpr int DK = D / 16;          // k-steps of the logit contraction
     static constexpr int DT = D / 32;          // 32-column tiles of the value contraction
     static constexpr int KS = D + 8;           // row stride of the q / K' / V' copies in LDS (bf16)
+    // Keys per K/V tile and sweep step, in 32-key halves.  (64-key tiles at head_dim 64, so that a step
+    // holds 16 MFMAs per wavefront as at head_dim 128, measured the same forward time as 32-key tiles at
+    // B2 H8 N2048 w 512/32 and cost 90 registers: 32 everywhere.)
+    static constexpr int TK = 32;
+    static constexpr int NSUB = TK / 32;
+    // Head dims up to 64: every wavefront keeps the running softmax state and the output accumulator
+    // of its units in registers (32 more at head_dim 64) and the eight are merged once at the end,
+    // instead of a fold through LDS with three barriers after every round of eight units.
+    static constexpr bool NOFOLD = D <= 64;
     // A K or V tile in LDS is written by direct global->LDS loads: one wavefront instruction
     // fills a group of RPW rows (1 KB), lane L putting the 16-byte chunk L / RPW of row
     // L % RPW at byte 16 * L.  Groups lie GROUP bytes apart.  Row operand reads and
@@ -61,7 +73,7 @@ struct Cfg {
     // byte offset of row r of a tile (chunk 0)
     static constexpr int row_off(int r) { return (r / RPW) * GROUP + (r % RPW) * 16; }
     static constexpr int GROUP = 1024 + 16 * RPW;           // bytes
-    static constexpr int NGROUP = TJ / RPW;
+    static constexpr int NGROUP = TK / RPW;
     static constexpr int TILE_BYTES = NGROUP * GROUP;
     static constexpr int STAGE = TILE_BYTES;                // bf16 elements of one stage = K tile + V tile
     static constexpr int SS = D + 8;                        // slab row stride (bf16)
@@ -96,6 +108,18 @@ struct Cfg {
 // left = 1, starts its accumulator from that pair and handles delta < w2 in full rounds.
 constexpr int MODE_FAST = 0, MODE_SAFE = 1, MODE_LEFT = 2;
 constexpr int PREPASS_MIN_WORKGROUPS = 768;      // three workgroups per CU
+
+// Transposed V operand reads of a whole tile, item I of N = (32-key half h, 32-column block dt,
+// k-step ks): rows 32h + 16ks + {0..7, 8..15} of columns 32dt .. 32dt+31, into vh[2I], vh[2I+1].
+template <class C, int I, int N, int M>
+__device__ __forceinline__ void issue_v_all(uint32_t addr, lds_half_operand (&vh)[M]) {
+    if constexpr (I < N) {
+        constexpr int h = I / (2 * C::DT), dt = (I / 2) % C::DT, ks = I % 2;
+        constexpr int base = dt * 64 * C::RPW;
+        lds_tr_issue<base + C::row_off(32 * h + 16 * ks), base + C::row_off(32 * h + 16 * ks + 8)>(addr, vh[2 * I], vh[2 * I + 1]);
+        issue_v_all<C, I + 1, N>(addr, vh);
+    }
+}
 
 // SIDE: the K' and V' rows the block's deltas reach are copied to LDS (they fit); otherwise
 // they are read from global memory where they are needed.
@@ -149,6 +173,7 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
     const uint16_t* v1p = (const uint16_t*)p.v1.p + p.v1.off(b, 0, h);
     const uint16_t* v2p = (const uint16_t*)p.v2.p + p.v2.off(b, 0, h);
 
+    constexpr int TJ = C::TK;                    // keys per tile in this kernel
     const int jt_lo = (i0_wg - w1 > 0 ? i0_wg - w1 : 0) / TJ;
     const int jt_hi = LEFT ? (i0_wg + FW * BQ - 1 < N - 1 ? i0_wg + FW * BQ - 1 : N - 1) / TJ : i_last / TJ;
     const int nt = jt_hi - jt_lo + 1;
@@ -301,13 +326,24 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
         ++g;
     };
 
+    // (NOFOLD) this wavefront's running result over its units: reference exponent and sum of every
+    // row, output accumulator in the layout of the value MFMAs' result
+    float Mw = -INFINITY, Lw = 0.f;
+    floatx16 wacc[C::NOFOLD ? C::DT : 1];
+    if constexpr (C::NOFOLD) {
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) wacc[dt][v] = 0.f;
+    }
+
     for (int round = 0; round < nrounds; ++round) {
         const int delta = LEFT ? w2 : round * FW + wave;
         const bool ok = LEFT ? (i0 < N && i_last >= w2) : delta < n_units;
         // The unit starts from the query's running reference point (finite from the second
         // round on, or from the first where the pre-pass ran), so only then it looks for maxima.
         float m = -INFINITY, l = 0.f;
-        if constexpr (!LEFT) m = ok ? fin_m[ln] : -INFINITY;
+        if constexpr (!LEFT) m = C::NOFOLD ? Mw : (ok ? fin_m[ln] : -INFINITY);
         floatx16 racc[C::DT];
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
@@ -382,41 +418,37 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             };
             constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;      // operand strides of a k-step / a 32-column block
             auto stage_addr = [&](int st) { return smem_addr + (uint32_t)st * (uint32_t)(C::STAGE * 2); };
-            auto logit_mfmas = [&](uint32_t ks_addr, floatx16 c) -> floatx16 {
+            constexpr uint32_t SUBB = C::row_off(32 % C::TK);                   // byte offset of a tile's second 32-key half
+            // logits of the 32-key half `h` of the tile at ks_addr
+            auto logit_mfmas = [&](uint32_t ks_addr, int h, floatx16 c) -> floatx16 {
 #pragma unroll
                 for (int kk = 0; kk < C::DK; ++kk) {
-                    const X8 ka = lds_read_x8<X8>(ks_addr + k_lane + kk * KKB);
+                    const X8 ka = lds_read_x8<X8>(ks_addr + k_lane + h * SUBB + kk * KKB);
                     c = E::mfma(ka, qf[kk], c, 0, 0, 0);
                 }
                 return c;
             };
-            // all transposed V operand reads of a tile (opaque reads, settled before use)
-            auto issue_v = [&](uint32_t vt_addr, lds_half_operand (&vh)[4 * C::DT]) {
-                constexpr int R8 = C::row_off(8), R16 = C::row_off(16), R24 = C::row_off(24);
-                lds_tr_issue<0, R8>(vt_addr, vh[0], vh[1]);
-                lds_tr_issue<R16, R24>(vt_addr, vh[2], vh[3]);
-                if constexpr (C::DT >= 2) {
-                    lds_tr_issue<1 * DTB, 1 * DTB + R8>(vt_addr, vh[4], vh[5]);
-                    lds_tr_issue<1 * DTB + R16, 1 * DTB + R24>(vt_addr, vh[6], vh[7]);
-                }
-                if constexpr (C::DT == 4) {
-                    lds_tr_issue<2 * DTB, 2 * DTB + R8>(vt_addr, vh[8], vh[9]);
-                    lds_tr_issue<2 * DTB + R16, 2 * DTB + R24>(vt_addr, vh[10], vh[11]);
-                    lds_tr_issue<3 * DTB, 3 * DTB + R8>(vt_addr, vh[12], vh[13]);
-                    lds_tr_issue<3 * DTB + R16, 3 * DTB + R24>(vt_addr, vh[14], vh[15]);
-                }
+            // all transposed V operand reads of a tile (opaque reads, settled before use):
+            // vh[((h * DT + dt) * 2 + ks) * 2 + {0, 1}] = the two halves of the operand of half h,
+            // 32-column block dt, k-step ks
+            auto issue_v = [&](uint32_t vt_addr, lds_half_operand (&vh)[4 * C::DT * C::NSUB]) {
+                issue_v_all<C, 0, 2 * C::DT * C::NSUB>(vt_addr, vh);
             };
+            // value MFMAs of a whole tile: w[2 * h + ks] = the weights of half h, k-step ks
             auto value_mfmas = [&](uint32_t vt_addr, const X8* w) {
-                lds_half_operand vh[4 * C::DT];
+                lds_half_operand vh[4 * C::DT * C::NSUB];
                 issue_v(vt_addr, vh);
                 lds_settle(vh);
 #pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt)
+                for (int h = 0; h < C::NSUB; ++h)
 #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const X8 va = lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
-                        racc[dt] = E::mfma(va, w[ks], racc[dt], 0, 0, 0);
-                    }
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks) {
+                            const int x = ((h * C::DT + dt) * 2 + ks) * 2;
+                            const X8 va = lds_join<X8>(vh[x], vh[x + 1]);
+                            racc[dt] = E::mfma(va, w[2 * h + ks], racc[dt], 0, 0, 0);
+                        }
             };
 
             // Mask of a tile as the C operand of its logit MFMAs: -m where the key is inside
@@ -440,22 +472,25 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             if (SAFE) {
                 // ---- repair pass: the reference point follows the maxima on every tile ----
                 for (int s = 0; s < nt; ++s) {
-                    const int j0 = (jt_lo + s) * TJ;
                     begin_step(s);
                     const uint32_t Ks = stage_addr(buf);
                     const bool plain = tile_plain(s);
-                    const int hi = i - j0 - 4 * hf, lo = hi - w1;
-                    floatx16 t;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) t[v] = 0.f;
-                    t = logit_mfmas(Ks, t);
+                    floatx16 t[C::NSUB];
                     float mx = -INFINITY;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int c = 8 * (v >> 2) + (v & 3);
-                        const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
-                        t[v] = valid ? t[v] : -INFINITY;
-                        mx = fmaxf(mx, t[v]);
+                    for (int h = 0; h < C::NSUB; ++h) {
+                        const int j0 = (jt_lo + s) * TJ + 32 * h;
+                        const int hi = i - j0 - 4 * hf, lo = hi - w1;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) t[h][v] = 0.f;
+                        t[h] = logit_mfmas(Ks, h, t[h]);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = 8 * (v >> 2) + (v & 3);
+                            const bool valid = plain | (row_ok & (c <= hi) & (c >= lo));
+                            t[h][v] = valid ? t[h][v] : -INFINITY;
+                            mx = fmaxf(mx, t[h][v]);
+                        }
                     }
                     mx = fmaxf(mx, other_half(mx));
                     const float m_new = fmaxf(m, mx);
@@ -467,12 +502,15 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) racc[dt][v] *= alpha;
+                    X8 pb[2 * C::NSUB];
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) t[v] -= m_use;
-                    X8 pb[2];
-                    float rs;
-                    weights(t, pb, rs);
-                    l += rs;
+                    for (int h = 0; h < C::NSUB; ++h) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) t[h][v] -= m_use;
+                        float rs;
+                        weights(t[h], pb + 2 * h, rs);
+                        l += rs;
+                    }
                     value_mfmas(Ks + C::TILE_BYTES + v_lane, pb);
                     advance();
                 }
@@ -485,18 +523,21 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     advance();
                 }
                 if (__builtin_amdgcn_ballot_w64(m == -INFINITY) != 0) {
-                    const int j0 = (jt_lo + ws0) * TJ;
-                    const int hi = i - j0 - 4 * hf, lo = hi - w1;
-                    floatx16 t;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) t[v] = 0.f;
-                    t = logit_mfmas(stage_addr(buf), t);
                     float mx = -INFINITY;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int c = 8 * (v >> 2) + (v & 3);
-                        const bool valid = row_ok & (c <= hi) & (c >= lo);
-                        mx = fmaxf(mx, valid ? t[v] : -INFINITY);
+                    for (int h = 0; h < C::NSUB; ++h) {
+                        const int j0 = (jt_lo + ws0) * TJ + 32 * h;
+                        const int hi = i - j0 - 4 * hf, lo = hi - w1;
+                        floatx16 t;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) t[v] = 0.f;
+                        t = logit_mfmas(stage_addr(buf), h, t);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = 8 * (v >> 2) + (v & 3);
+                            const bool valid = row_ok & (c <= hi) & (c >= lo);
+                            mx = fmaxf(mx, valid ? t[v] : -INFINITY);
+                        }
                     }
                     mx = fmaxf(mx, other_half(mx));
                     if (m == -INFINITY) m = (mx == -INFINITY) ? 0.f : mx;
@@ -507,11 +548,13 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 // ---- two-stage software pipeline over the tiles: step t issues the logit MFMAs
                 // of tile t between the softmax instructions of tile t-1, then the value MFMAs
                 // of tile t-1; the shifted logits of tile t wait in registers for step t+1.
-                floatx16 sh_a, sh_b;
+                floatx16 sh_a[C::NSUB], sh_b[C::NSUB];
                 {
-                    const floatx16 c0 = tile_plain(ws0) ? negm : masked_c((jt_lo + ws0) * TJ);
+                    const bool plain0 = tile_plain(ws0);
                     begin_step(ws0);
-                    sh_a = logit_mfmas(stage_addr(buf), c0);
+#pragma unroll
+                    for (int h = 0; h < C::NSUB; ++h)
+                        sh_a[h] = logit_mfmas(stage_addr(buf), h, plain0 ? negm : masked_c((jt_lo + ws0) * TJ + 32 * h));
                 }
                 uint32_t vt_prev = stage_addr(buf) + (uint32_t)C::TILE_BYTES + v_lane;
                 advance();
@@ -520,27 +563,40 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 // two steps of the kernel do).  Both are compile-time so that a step is one
                 // basic block: the request's scalar arithmetic and the loads then sit between the
                 // MFMAs instead of in front of them, where both wavefronts of a SIMD would wait.
-                auto step = [&](int s, const floatx16& prev, floatx16& cur, auto PLAIN_TAG, auto DMA_TAG) {
+                auto step = [&](int s, const floatx16 (&prev)[C::NSUB], floatx16 (&cur)[C::NSUB], auto PLAIN_TAG, auto DMA_TAG) {
                     constexpr bool PLAIN = decltype(PLAIN_TAG)::value, DMA = decltype(DMA_TAG)::value;
                     const uint32_t ks_addr = stage_addr(buf);
-                    X8 ka[C::DK];
+                    X8 ka[C::NSUB][C::DK];
 #pragma unroll
-                    for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_x8<X8>(ks_addr + k_lane + kk * KKB);
+                    for (int h = 0; h < C::NSUB; ++h)
+#pragma unroll
+                        for (int kk = 0; kk < C::DK; ++kk) ka[h][kk] = lds_read_x8<X8>(ks_addr + k_lane + h * SUBB + kk * KKB);
                     // the reference point (and, on the window-edge tiles, the mask) is the
                     // C operand of the first logit MFMA
-                    if constexpr (PLAIN) cur = E::mfma(ka[0], qf[0], negm, 0, 0, 0);
-                    else cur = E::mfma(ka[0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
+                    if constexpr (PLAIN) cur[0] = E::mfma(ka[0][0], qf[0], negm, 0, 0, 0);
+                    else cur[0] = E::mfma(ka[0][0], qf[0], masked_c((jt_lo + s) * TJ), 0, 0, 0);
                     if constexpr (DMA) dma_next();
-                    lds_half_operand vh[4 * C::DT];
+                    lds_half_operand vh[4 * C::DT * C::NSUB];
                     issue_v(vt_prev, vh);
-                    X8 pb[2];
-                    float rs;
+                    X8 pb[2 * C::NSUB];
 #pragma unroll
                     for (int kk = 1; kk < C::DK; ++kk)
-                        cur = E::mfma(ka[kk], qf[kk], cur, 0, 0, 0);
-                    weights(prev, pb, rs);
-                    l += rs;
-                    bad |= !(rs < E::WEIGHT_LIMIT);
+                        cur[0] = E::mfma(ka[0][kk], qf[kk], cur[0], 0, 0, 0);
+#pragma unroll
+                    for (int h = 1; h < C::NSUB; ++h) {
+                        if constexpr (PLAIN) cur[h] = E::mfma(ka[h][0], qf[0], negm, 0, 0, 0);
+                        else cur[h] = E::mfma(ka[h][0], qf[0], masked_c((jt_lo + s) * TJ + 32 * h), 0, 0, 0);
+#pragma unroll
+                        for (int kk = 1; kk < C::DK; ++kk)
+                            cur[h] = E::mfma(ka[h][kk], qf[kk], cur[h], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int h = 0; h < C::NSUB; ++h) {
+                        float rs;
+                        weights(prev[h], pb + 2 * h, rs);
+                        l += rs;
+                        bad |= !(rs < E::WEIGHT_LIMIT);
+                    }
                     asm volatile("" : "+v"(pb[0]));              // (the wait below stays behind the first weights)
                     lds_settle(vh);
                     // The barrier stands in front of the value MFMAs: they only read registers.
@@ -550,16 +606,20 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     buf = (buf + 1) & (C::NSTAGE - 1);
                     ++g;
 #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
+                    for (int h = 0; h < C::NSUB; ++h)
 #pragma unroll
-                        for (int dt = 0; dt < C::DT; ++dt) {
-                            const X8 va = lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]);
-                            racc[dt] = E::mfma(va, pb[ks], racc[dt], 0, 0, 0);
-                        }
+                        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                            for (int dt = 0; dt < C::DT; ++dt) {
+                                const int x = ((h * C::DT + dt) * 2 + ks) * 2;
+                                const X8 va = lds_join<X8>(vh[x], vh[x + 1]);
+                                racc[dt] = E::mfma(va, pb[2 * h + ks], racc[dt], 0, 0, 0);
+                            }
                     // the softmax arithmetic is spread over the MFMAs of the step
-                    constexpr int PER = (36 + C::DK + 2 * C::DT - 1) / (C::DK + 2 * C::DT);
+                    constexpr int NMFMA = C::NSUB * (C::DK + 2 * C::DT);
+                    constexpr int PER = (36 * C::NSUB + NMFMA - 1) / NMFMA;
 #pragma unroll
-                    for (int x = 0; x < C::DK + 2 * C::DT; ++x) {
+                    for (int x = 0; x < NMFMA; ++x) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
                         __builtin_amdgcn_sched_group_barrier(0x402, PER, 0);             // a slice of VALU / exp
                     }
@@ -576,12 +636,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     }
                     if (s <= to_dma) {
                         step(s, sh_a, sh_b, PLAIN_TAG, std::true_type{});
-                        sh_a = sh_b;
+#pragma unroll
+                        for (int h = 0; h < C::NSUB; ++h) sh_a[h] = sh_b[h];
                         ++s;
                     }
                     for (; s <= to; ++s) {               // the last two steps of the kernel
                         step(s, sh_a, sh_b, std::false_type{}, std::false_type{});
-                        sh_a = sh_b;
+#pragma unroll
+                        for (int h = 0; h < C::NSUB; ++h) sh_a[h] = sh_b[h];
                     }
                 };
                 // window-edge tiles, tiles that need no mask, window-edge tiles
@@ -592,11 +654,14 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                     run(p_hi, std::true_type{});
                 }
                 run(ws1, std::false_type{});
-                X8 pb[2];
-                float rs;
-                weights(sh_a, pb, rs);
-                l += rs;
-                bad |= !(rs < E::WEIGHT_LIMIT);
+                X8 pb[2 * C::NSUB];
+#pragma unroll
+                for (int h = 0; h < C::NSUB; ++h) {
+                    float rs;
+                    weights(sh_a[h], pb + 2 * h, rs);
+                    l += rs;
+                    bad |= !(rs < E::WEIGHT_LIMIT);
+                }
                 value_mfmas(vt_prev, pb);
                 for (int s2 = ws1 + 1; s2 < nt; ++s2) {   // (pre-pass) tiles after this wavefront's window
                     begin_step(s2);
@@ -635,6 +700,57 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
                 }
             }
             return;
+        }
+
+        if constexpr (C::NOFOLD) {
+            // ---- the unit joins the wavefront's running result: O += e^(m-M) * (v2 + bias) * R ----
+            if (ok) {
+                const int tid_u = recompute_here(threadIdx.x);
+                const int ln_u = tid_u & 31, hf_u = (tid_u >> 5) & 1;
+                const uint16_t* vrow;
+                if constexpr (SIDE) {
+                    vrow = v2_s + (ln_u + w2 - delta) * C::KS + 4 * hf_u;
+                } else {
+                    const int iq = i0 + ln_u < N ? i0 + ln_u : N - 1;
+                    vrow = v2p + (int64_t)(iq - delta > 0 ? iq - delta : 0) * p.v2.sn + 4 * hf_u;
+                }
+                uint2 vx[4 * C::DT];
+#pragma unroll
+                for (int e = 0; e < 4 * C::DT; ++e) vx[e] = *(const uint2*)(vrow + (e >> 2) * 32 + 8 * (e & 3));
+                const float lt = l + other_half(l);
+                const bool row_has = (i0 + ln_u < N) & (i0 + ln_u >= delta);
+                // The fast kernel keeps a unit's reference point fixed, and every unit after the wavefront's
+                // first starts from the running one: all weights are 1.  The repair kernel moves it.
+                float a = 1.f, c = 1.f;
+                if (SAFE) {
+                    const float Mn = fmaxf(Mw, m), Mu = Mn == -INFINITY ? 0.f : Mn;
+                    a = fast_exp2(Mw - Mu);
+                    c = fast_exp2(m - Mu);
+                    Mw = Mn;
+                } else {
+                    Mw = row_has ? m : Mw;           // (a row without a key in this unit keeps its state)
+                }
+                Lw = Lw * a + lt * c;
+                const float vb = p.v2_bias;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const uint2 x = vx[4 * dt + g4];
+                        if (SAFE) {
+                            wacc[dt][4 * g4 + 0] = wacc[dt][4 * g4 + 0] * a + c * racc[dt][4 * g4 + 0] * (E::lo(x.x) + vb);
+                            wacc[dt][4 * g4 + 1] = wacc[dt][4 * g4 + 1] * a + c * racc[dt][4 * g4 + 1] * (E::hi(x.x) + vb);
+                            wacc[dt][4 * g4 + 2] = wacc[dt][4 * g4 + 2] * a + c * racc[dt][4 * g4 + 2] * (E::lo(x.y) + vb);
+                            wacc[dt][4 * g4 + 3] = wacc[dt][4 * g4 + 3] * a + c * racc[dt][4 * g4 + 3] * (E::hi(x.y) + vb);
+                        } else {
+                            wacc[dt][4 * g4 + 0] += racc[dt][4 * g4 + 0] * (E::lo(x.x) + vb);
+                            wacc[dt][4 * g4 + 1] += racc[dt][4 * g4 + 1] * (E::hi(x.x) + vb);
+                            wacc[dt][4 * g4 + 2] += racc[dt][4 * g4 + 2] * (E::lo(x.y) + vb);
+                            wacc[dt][4 * g4 + 3] += racc[dt][4 * g4 + 3] * (E::hi(x.y) + vb);
+                        }
+                    }
+            }
+            continue;
         }
 
         // ---- fold the round's units into the workgroup accumulator --------------
@@ -766,6 +882,70 @@ void mfma_fwd_kernel(Problem p, int nqb, int total, int left) {
             for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
         }
         __syncthreads();       // the stage buffers that served as slabs are requested again in the next steps
+    }
+
+    if constexpr (C::NOFOLD && !LEFT) {
+        // ---- merge the eight wavefronts (and the pre-pass partial) into the LDS accumulator ----
+        const int tid_m = recompute_here(threadIdx.x);
+        const int ln_m = tid_m & 31, hf_m = (tid_m >> 5) & 1;
+        const int aq = tid_m >> 4, ac = (tid_m & 15) * ACN;
+        if (hf_m == 0) {
+            xch_m[wave * BQ + ln_m] = Mw;
+            xch_l[wave * BQ + ln_m] = Lw;
+        }
+        __syncthreads();           // (also: every wavefront is done with the tile ring, which the sums go through)
+        const bool with_left = has_left && !SAFE;
+        auto reference = [&](int row) {
+            float mx = with_left ? lam_s[row] : -INFINITY;
+#pragma unroll
+            for (int w = 0; w < FW; ++w) mx = fmaxf(mx, xch_m[w * BQ + row]);
+            return mx;
+        };
+        // writer side: this wavefront's rows scaled to the common reference
+        const float Mrow = reference(ln_m);
+        const float cw = Mw == -INFINITY ? 0.f : fast_exp2(Mw - Mrow);
+        // reader side: this thread's slice of the accumulator
+        const float Mq = reference(aq), Mq_use = Mq == -INFINITY ? 0.f : Mq;
+        float Ln = 0.f;
+#pragma unroll
+        for (int w = 0; w < FW; ++w) {
+            const float mw = xch_m[w * BQ + aq];
+            Ln += mw == -INFINITY ? 0.f : xch_l[w * BQ + aq] * fast_exp2(mw - Mq_use);
+        }
+        float acc[ACN];
+        {
+            const float al = (with_left && lam_s[aq] > -INFINITY) ? fast_exp2(lam_s[aq] - Mq_use) : 0.f;
+            Ln += al;                                                     // the pre-pass partial has sum 1 at its reference
+#pragma unroll
+            for (int c = 0; c < ACN; ++c) acc[c] = with_left ? al * oacc[aq * C::OS + ac + c] : 0.f;
+        }
+        float* mbuf = (float*)smem_raw;                                   // [4][BQ][OS] fp32, over the tile ring
+        static_assert((size_t)4 * BQ * C::OS * 4 <= C::STAGE_BYTES, "the merge buffer lies over the tile ring");
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            if ((wave >> 2) == pass) {
+                float* mrow = mbuf + ((wave & 3) * BQ + ln_m) * C::OS + 4 * hf_m;
+#pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4)
+                        *(float4*)(mrow + dt * 32 + 8 * g4) = make_float4(cw * wacc[dt][4 * g4], cw * wacc[dt][4 * g4 + 1],
+                                                                          cw * wacc[dt][4 * g4 + 2], cw * wacc[dt][4 * g4 + 3]);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+#pragma unroll
+                for (int c = 0; c < ACN; ++c) acc[c] += mbuf[(w * BQ + aq) * C::OS + ac + c];
+            __syncthreads();
+        }
+#pragma unroll
+        for (int c = 0; c < ACN; ++c) oacc[aq * C::OS + ac + c] = acc[c];
+        if ((tid_m & 15) == 0) {
+            fin_m[aq] = Mq;
+            fin_l[aq] = Ln;
+        }
+        __syncthreads();
     }
 
     // ---- normalise and store ------------------------------------------------------

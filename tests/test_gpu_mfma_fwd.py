@@ -100,7 +100,8 @@ def test_auto_dispatch_takes_mfma_for_bf16_d64_d128():
     assert lib.sa2_uses_mfma(2, 2048, 8, 64, 512, 32, _lib.SA2_BF16) == 1
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_BF16) == 1
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F16) == 1
-    assert lib.sa2_uses_mfma(1, 128, 2, 64, 32, 16, _lib.SA2_F32) == 0
+    assert lib.sa2_uses_mfma(1, 128, 2, 64, 32, 16, _lib.SA2_F32) == 1      # (the fp32 MFMA kernels)
+    assert lib.sa2_uses_mfma(1, 128, 2, 256, 32, 16, _lib.SA2_F32) == 0
     assert lib.sa2_uses_mfma(1, 128, 2, 32, 32, 16, _lib.SA2_BF16) == 1
     assert lib.sa2_uses_mfma(1, 128, 2, 48, 32, 16, _lib.SA2_BF16) == 0
     inp = make_inputs(1, 96, 2, 64, seed=1, dtype=torch.bfloat16, with_dout=False)
