@@ -96,8 +96,9 @@ void* static_workspace() {
 
 size_t dsum_bytes(int B, int N, int H) { return align_up((size_t)B * H * N * sizeof(float), 256); }
 
-// Which kernels a call takes: the fp32 FMA kernels, the 16-bit MFMA kernels, or the fp32 MFMA kernels.
-enum KernelPath { PATH_GENERIC, PATH_MFMA16, PATH_MFMA32 };
+// Which kernels a call takes: the fp32 FMA kernels, the tuned 16-bit MFMA kernels (head_dim 32, 64, 128), the
+// 16-bit MFMA kernels for head_dim 256, or the fp32 MFMA kernels.
+enum KernelPath { PATH_GENERIC, PATH_MFMA16, PATH_WIDE16, PATH_MFMA32 };
 
 KernelPath pick_path(const Problem& p, int dtype, unsigned flags, bool backward, int* status) {
     *status = SA2_OK;
@@ -112,6 +113,8 @@ KernelPath pick_path(const Problem& p, int dtype, unsigned flags, bool backward,
                                   : mfma_supported(p.B, p.N, p.H, p.D, p.w1, p.w2, dtype)) &&
                         mfma_layout_ok(p, backward);
         if (ok) path = PATH_MFMA16;
+        else if ((backward ? wide_bwd_supported(p.D, p.w2, dtype) : wide_supported(p.D, dtype)) && mfma_layout_ok(p, backward))
+            path = PATH_WIDE16;
     }
     if (path == PATH_GENERIC && (flags & SA2_FLAG_FORCE_MFMA)) *status = SA2_ERR_UNSUPPORTED;
     return path;
@@ -143,7 +146,8 @@ const char* sa2_strerror(int status) {
 
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype) {
     if (check_dims(B, N, H, D, w1, w2, dtype, 1) != SA2_OK) return 0;
-    return (mfma_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype) || f32_mfma_supported(D, dtype)) ? 1 : 0;
+    return (mfma_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype) || wide_supported(D, dtype) ||
+            f32_mfma_supported(D, dtype)) ? 1 : 0;
 }
 
 int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
@@ -175,6 +179,7 @@ int sa2_forward(const void* q, const void* k1, const void* k2, const void* v1, c
     const KernelPath path = pick_path(p, dtype, flags, false, &rc);
     if (rc != SA2_OK) return rc;
     return path == PATH_MFMA16 ? launch_mfma_fwd(p, dtype, st)
+           : path == PATH_WIDE16 ? launch_wide_fwd(p, dtype, st)
            : path == PATH_MFMA32 ? launch_f32_mfma_fwd(p, st) : launch_generic_fwd(p, dtype, st);
 }
 
@@ -183,6 +188,10 @@ size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int d
     size_t scratch = generic_bwd_scratch_bytes(B, N, H, D, w1, w2);
     if (!(flags & SA2_FLAG_FORCE_GENERIC) && mfma_bwd_supported(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N), dtype)) {
         const size_t m = mfma_bwd_scratch_bytes(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N));
+        if (m > scratch) scratch = m;
+    }
+    if (!(flags & SA2_FLAG_FORCE_GENERIC) && wide_bwd_supported(D, reach(w2, 1, N), dtype)) {
+        const size_t m = wide_bwd_scratch_bytes(B, N, H, D, reach(w2, 1, N));
         if (m > scratch) scratch = m;
     }
     if (!(flags & SA2_FLAG_FORCE_GENERIC) && f32_mfma_bwd_supported(D, reach(w2, 1, N), dtype)) {
@@ -238,6 +247,7 @@ int sa2_backward(const void* q, const void* k1, const void* k2, const void* v1, 
     const KernelPath path = pick_path(p, dtype, flags, true, &rc);
     if (rc != SA2_OK) return rc;
     return path == PATH_MFMA16 ? launch_mfma_bwd(p, dtype, st)
+           : path == PATH_WIDE16 ? launch_wide_bwd(p, dtype, st)
            : path == PATH_MFMA32 ? launch_f32_mfma_bwd(p, st) : launch_generic_bwd(p, dtype, st);
 }
 

@@ -72,7 +72,8 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_BF16) == 1
     assert lib.sa2_uses_mfma(1, 8192, 16, 128, 512, 32, _lib.SA2_F32) == 1      # the fp32 MFMA kernels
     assert lib.sa2_uses_mfma(1, 8192, 16, 256, 512, 32, _lib.SA2_F32) == 0
-    assert lib.sa2_uses_mfma(1, 8192, 16, 256, 512, 32, _lib.SA2_BF16) == 0
+    assert lib.sa2_uses_mfma(1, 8192, 16, 256, 512, 32, _lib.SA2_BF16) == 1     # the head_dim 256 MFMA kernels
+    assert lib.sa2_uses_mfma(1, 8192, 16, 192, 512, 32, _lib.SA2_BF16) == 0
 
 
 def test_forced_mfma_refuses_layouts_its_loads_cannot_take(lib):
