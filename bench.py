@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the 2-simplicial attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c2f32]
 
 A step is one forward + backward pass of the operator over one batch of
 synthetic input that is already resident in HBM (iid normal, seeded, bf16).
 The default workload is the headline configuration: bf16, B=1 H=16 N=8192 D=128,
-w1=512 w2=32.  Prints ONE JSON line:
+w1=512 w2=32.  Workloads c1 (fp32 B=1 H=2 N=128 D=64 w 32/16, the forward-only plumbing
+configuration) and c2f32 (fp32 tensors at the shape of c2) run on the fp32 MFMA kernels and are
+priced against the fp32 matrix peak.  Prints ONE JSON line:
 
   metric/value   forward+backward algorithmic TFLOP/s: 16*D*T flops per step,
                  T = number of valid (i,j,k) triples (matmul flops only, 2 per
@@ -49,11 +51,13 @@ BF16_FLOP_PER_CLK_PER_CU = 4096
 
 WORKLOADS = {
     # name: (B, N, H, D, w1, w2, seed, qk_std)
+    "c1": (1, 128, 2, 64, 32, 16, 0, 1.0),
     "c2": (2, 2048, 8, 64, 512, 32, 1, 1.0),
     "c4": (1, 8192, 16, 128, 512, 32, 3, 1.0),
     "c5": (1, 32768, 8, 128, 1024, 64, 4, 0.5),
+    "c2f32": (2, 2048, 8, 64, 512, 32, 1, 1.0),
 }
-
+FP32_WORKLOADS = ("c1", "c2f32")
 
 
 def profile_keys():
@@ -76,14 +80,14 @@ def count_triples(B, N, H, w1, w2):
     return B * H * sum((min(i, w1) + 1) * (min(i, w2) + 1) for i in range(N))
 
 
-def make_inputs(B, N, H, D, seed, qk_std, device):
+def make_inputs(B, N, H, D, seed, qk_std, device, dtype=torch.bfloat16):
     g = torch.Generator().manual_seed(seed)
     out = []
     for t in range(6):
         x = torch.randn(B, N, H, D, generator=g, dtype=torch.float32)
         if t < 3:
             x = x * qk_std
-        out.append(x.to(torch.bfloat16).to(device))
+        out.append(x.to(dtype).to(device))
     return out
 
 
@@ -219,7 +223,7 @@ def cpu_reference_literal(target_iterations, target_name):
     }
 
 
-def cpu_baseline(name, cfg, budget_rows):
+def cpu_baseline(name, cfg, budget_rows, fp32=False):
     """Times the CPU oracle forward + autograd on `budget_rows` steady-state
     query rows of the workload (all batches and heads) and scales by the triple
     count.  Returns the JSON object."""
@@ -231,7 +235,8 @@ def cpu_baseline(name, cfg, budget_rows):
         x = torch.randn(B, N, H, D, generator=g, dtype=torch.float32)
         if t < 3:
             x = x * qk_std
-        tens.append(x.to(torch.bfloat16).float())
+        tens.append(x if fp32 else x.to(torch.bfloat16).float())
+    budget_rows = min(budget_rows, N)
     r0 = min(N - budget_rows, max(w1, w2) + 64)
     r0 = max(r0, 0)
     r1 = min(N, r0 + budget_rows)
@@ -274,14 +279,19 @@ def main():
 
     cfg = WORKLOADS[args.workload]
     B, N, H, D, w1, w2, seed, qk_std = cfg
+    fp32 = args.workload in FP32_WORKLOADS
+    dtype_name, code = ("fp32", _lib.SA2_F32) if fp32 else ("bf16", _lib.SA2_BF16)
+    # published dense matrix peak of the arithmetic type the kernels compute in
+    PEAK_TFLOPS = PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS
     dev = torch.device("cuda:0")
     props = torch.cuda.get_device_properties(0)
-    q, k1, k2, v1, v2, dout = make_inputs(B, N, H, D, seed, qk_std, dev)
+    q, k1, k2, v1, v2, dout = make_inputs(B, N, H, D, seed, qk_std, dev, torch.float32 if fp32 else torch.bfloat16)
     T = count_triples(B, N, H, w1, w2)
     fwd_flops, bwd_flops = 4.0 * D * T, 12.0 * D * T
     E = B * N * H * D
-    fwd_bytes = 6 * E * 2 + 4 * B * H * N                  # read q,k1,k2,v1,v2; write O, LSE
-    bwd_bytes = 12 * E * 2 + 12 * B * H * N                # read 5 inputs, O, dO; write 5 grads; LSE, D
+    esz = 4 if fp32 else 2
+    fwd_bytes = 6 * E * esz + 4 * B * H * N                # read q,k1,k2,v1,v2; write O, LSE
+    bwd_bytes = 12 * E * esz + 12 * B * H * N              # read 5 inputs, O, dO; write 5 grads; LSE, D
 
     if args.counters_only:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -345,31 +355,34 @@ def main():
                                                         needs=(False, True, False, True, False)), ksteps, 2) - rowdot_ms
     bwd_rest_ms = time_gpu(lambda: sa.simplicial_backward(q, k1, k2, v1, v2, out, lse, dout, w1, w2,
                                                           needs=(True, False, True, False, True)), ksteps, 2) - rowdot_ms
-    mfma = bool(lib.sa2_uses_mfma(B, N, H, D, w1, w2, _lib.SA2_BF16))
+    mfma = bool(lib.sa2_uses_mfma(B, N, H, D, w1, w2, code))
     # Algorithmic flops per launch: forward 4*D*T; the backward's 12*D*T split evenly between its
     # two MFMA kernels (each owns two output contractions, 4*D*T, and half of the S / dP
     # recomputation that the pair shares, 2*D*T).
     half_bwd = bwd_flops / 2
     keys, key_sources = profile_keys()
     wl = args.workload
+    if fp32:
+        labels = ("f32_fwd_kernel<%d> (v_mfma_f32_32x32x2_f32)" % D, 1, "f32_bwd_kv_kernel<%d> (dK, dV)" % D, 1,
+                  "f32_bwd_kp_kernel<%d> + f32_dq_sum_kernel (dQ, dK', dV')" % D, 2)
+    else:
+        labels = ("mfma_fwd_kernel<%d> (pre-pass + fast kernel + repair launch)" % D, 3, "mfma_bwd_kv_kernel<%d> (dK, dV)" % D, 1,
+                  "mfma_bwd_kp_kernel<%d> (pre-pass + main) + dq_sum (dQ, dK', dV')" % D, 3)
     kernels = {
-        "forward": {"kernel": "mfma_fwd_kernel<%d> (pre-pass + fast kernel + repair launch)" % D, "ms": fwd_ms,
-                    "flops": fwd_flops, "launches": 3},
-        "backward_k_side": {"kernel": "mfma_bwd_kv_kernel<%d> (dK, dV)" % D, "ms": bwd_k1_ms, "flops": half_bwd,
-                            "launches": 1},
-        "backward_kprime_side": {"kernel": "mfma_bwd_kp_kernel<%d> (pre-pass + main) + dq_sum (dQ, dK', dV')" % D, "ms": bwd_rest_ms,
-                                 "flops": half_bwd, "launches": 3},
+        "forward": {"kernel": labels[0], "ms": fwd_ms, "flops": fwd_flops, "launches": labels[1]},
+        "backward_k_side": {"kernel": labels[2], "ms": bwd_k1_ms, "flops": half_bwd, "launches": labels[3]},
+        "backward_kprime_side": {"kernel": labels[4], "ms": bwd_rest_ms, "flops": half_bwd, "launches": labels[5]},
     }
     for name, k in kernels.items():
         k["tflops"] = k["flops"] / k["ms"] / 1e9
-        k["frac_bf16_peak"] = k["tflops"] / PEAK_BF16_TFLOPS
+        k["frac_bf16_peak"] = k["tflops"] / PEAK_TFLOPS              # (of the fp32 matrix peak for the fp32 workloads)
         k["mfma_busy"] = keys.get((wl, name, "mfma_busy"))          # rocprofv3, from profiles/
         k["traffic"] = keys.get((wl, name, "traffic_bytes"))
     kernels["forward"]["hbm_gbs"] = fwd_bytes / fwd_ms / 1e6
     kernels["forward"]["ms_in_step"] = fwd_in_step_ms
-    kernels["forward"]["frac_bf16_peak_in_step"] = fwd_flops / fwd_in_step_ms / 1e9 / PEAK_BF16_TFLOPS
+    kernels["forward"]["frac_bf16_peak_in_step"] = fwd_flops / fwd_in_step_ms / 1e9 / PEAK_TFLOPS
     kernels["backward"] = {"ms": bwd_all_ms, "tflops": bwd_flops / bwd_all_ms / 1e9, "hbm_gbs": bwd_bytes / bwd_all_ms / 1e6,
-                           "frac_bf16_peak": bwd_flops / bwd_all_ms / 1e9 / PEAK_BF16_TFLOPS}
+                           "frac_bf16_peak": bwd_flops / bwd_all_ms / 1e9 / PEAK_TFLOPS}
     kernels["backward"]["ms_in_step"] = bwd_in_step_ms
     kernels["rowdot"] = {"ms": rowdot_ms, "hbm_gbs": (4 * E + 4 * B * H * N) / rowdot_ms / 1e6}
 
@@ -380,11 +393,12 @@ def main():
     for cname, call, ms_call in (("forward", fwd_call, fwd_ms), ("backward", bwd_call, bwd_all_ms), ("step", step, ms_per_step)):
         clocks[cname] = observed_clock_mhz(call, ms_call)
     cus = props.multi_processor_count
-    peak_at = lambda mhz: cus * BF16_FLOP_PER_CLK_PER_CU * mhz * 1e6 / 1e12
+    flop_per_clk_per_cu = int(round(BF16_FLOP_PER_CLK_PER_CU * PEAK_TFLOPS / PEAK_BF16_TFLOPS))      # 4096 bf16, 256 fp32
+    peak_at = lambda mhz: cus * flop_per_clk_per_cu * mhz * 1e6 / 1e12
     clock = {"mhz": clocks, "method": "device cycle counter (60 ms spin kernel on a second stream) / event time",
              "peak_bf16_tflops_at_observed_clock": {k: peak_at(v) for k, v in clocks.items()},
-             "published_peak_bf16_tflops": PEAK_BF16_TFLOPS,
-             "published_peak_is": "%d CU x 2400 MHz x %d flop/clk/CU" % (cus, BF16_FLOP_PER_CLK_PER_CU)}
+             "published_peak_bf16_tflops": PEAK_TFLOPS,
+             "published_peak_is": "%d CU x 2400 MHz x %d flop/clk/CU (%s matrix)" % (cus, flop_per_clk_per_cu, dtype_name)}
     kernels["forward"]["frac_at_observed_clock"] = kernels["forward"]["tflops"] / peak_at(clocks["forward"])
     for name in ("backward_k_side", "backward_kprime_side", "backward"):
         kernels[name]["frac_at_observed_clock"] = kernels[name]["tflops"] / peak_at(clocks["backward"])
@@ -397,7 +411,7 @@ def main():
     roofline = {
         "bound": "mfma", "kernel": kernels[dominant]["kernel"], "group": dominant,
         "launches": kernels[dominant]["launches"],
-        "achieved": kernels[dominant]["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+        "achieved": kernels[dominant]["tflops"], "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": kernels[dominant]["frac_bf16_peak"],
         "traffic": kernels[dominant]["traffic"],
         "algorithmic_flops_per_launch": kernels[dominant]["flops"],
@@ -410,7 +424,7 @@ def main():
     }
     roofline_fwd = {
         "bound": "mfma", "kernel": kernels["forward"]["kernel"], "achieved": kernels["forward"]["tflops"],
-        "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": kernels["forward"]["frac_bf16_peak"],
+        "peak": PEAK_TFLOPS, "unit": "TFLOP/s", "frac": kernels["forward"]["frac_bf16_peak"],
         "frac_at_observed_clock": kernels["forward"]["frac_at_observed_clock"],
         "mfma_busy": kernels["forward"]["mfma_busy"], "traffic": kernels["forward"]["traffic"],
         "counters_from": key_sources.get(wl),
@@ -437,19 +451,20 @@ def main():
     roofline_fwd["frac_of_library_gemm_on_n01"] = roofline_fwd["achieved"] / gemm["n01"]
 
     line = {
-        "metric": "fwd+bwd TFLOP/s & %% bf16 MFMA peak, N=%d D=%d w1=%d w2=%d" % (N, D, w1, w2),
+        "metric": "fwd+bwd TFLOP/s & %% %s MFMA peak, N=%d D=%d w1=%d w2=%d" % (dtype_name, N, D, w1, w2),
         "value": (fwd_flops + bwd_flops) / ms_per_step / 1e9,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "wall_ms_per_step": wall_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "%s: bf16 fwd+bwd B=%d H=%d N=%d D=%d w1=%d w2=%d scale=1/sqrt(D)" % (
-                       args.workload, B, H, N, D, w1, w2),
+        "dtype": dtype_name, "data": "synthetic",
+        "config": {"workload": "%s: %s fwd+bwd B=%d H=%d N=%d D=%d w1=%d w2=%d scale=1/sqrt(D)" % (
+                       args.workload, dtype_name, B, H, N, D, w1, w2),
                    "triples": T, "flops_fwd": fwd_flops, "flops_bwd": bwd_flops,
                    "mfma_kernels": mfma, "device": props.name, "cus": cus,
                    "clock_mhz": clocks["step"]},
-        "frac_bf16_peak": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
+        "frac_bf16_peak": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / PEAK_TFLOPS,
+        "peak_tflops": PEAK_TFLOPS,
         "frac_bf16_peak_at_observed_clock": (fwd_flops + bwd_flops) / ms_per_step / 1e9 / peak_at(clocks["step"]),
         "clock": clock,
         "power": power,
@@ -458,7 +473,7 @@ def main():
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_rows)
+        line["cpu_baseline"] = cpu_baseline(args.workload, cfg, args.cpu_rows, fp32)
         line["cpu_reference_literal"] = cpu_reference_literal(T // (B * H), "%s forward" % args.workload)
     print(json.dumps(line))
 
