@@ -102,8 +102,12 @@ int launch_wide_bwd(const Problem& p, int dtype, hipStream_t st);
 bool kp_fits(int D, int w2);
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2);
 int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st);
-// K-side backward kernel (dK, dV) with paired wavefronts
+// K-side backward kernel (dK, dV) with paired wavefronts; for small grids it splits a key block's
+// query blocks over several workgroups, whose fp32 partial sums lie in the workspace behind the
+// K'-side part (kp_side_scratch_bytes)
 bool kv_fits(int D, int w2);
+size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1);
+size_t kp_side_scratch_bytes(int B, int N, int H, int D, int w2);
 int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st);
 
 }  // namespace sa2

@@ -621,11 +621,15 @@ bool mfma_bwd_supported(int B, int N, int H, int D, int w1, int w2, int dtype) {
     return D != 32 || (kp_fits(D, w2) && kv_fits(D, w2));
 }
 
-size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
-    (void)w1;
-    if (kp_fits(D, w2)) return kp_scratch_bytes(B, N, H, D, w2);
+// Workspace of the K'-side kernels (dQ partials, or the expanded-row arrays of the workspace kernels),
+// rounded up so that what follows it stays 256-byte aligned
+size_t kp_side_scratch_bytes(int B, int N, int H, int D, int w2) {
     const size_t one = (expanded_ws_bytes(B, N, H, D, w2) + 255) / 256 * 256;
-    return 2 * one;
+    return kp_fits(D, w2) ? (kp_scratch_bytes(B, N, H, D, w2) + 255) / 256 * 256 : 2 * one;
+}
+
+size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
+    return kp_side_scratch_bytes(B, N, H, D, w2) + (kv_fits(D, w2) ? kv_split_scratch_bytes(B, N, H, D, w1) : 0);
 }
 
 int launch_mfma_bwd(const Problem& p, int dtype, hipStream_t st) {

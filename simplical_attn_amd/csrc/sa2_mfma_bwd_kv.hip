@@ -1,7 +1,9 @@
 // MFMA backward for gfx950 (bf16 or fp16 elements), the K-side kernel: dK and dV.
 //
-// A workgroup owns 128 consecutive K/V rows, 32 per wavefront pair, resident in registers
-// as MFMA B operands.  It streams every unit of expanded rows that can see them: unit
+// A workgroup owns 128 consecutive K/V rows, 32 per wavefront pair (at head_dim 64, where the
+// registers allow it and the grid stays large enough: 256 rows, two 32-row blocks per pair, so
+// that a unit's forming, its operand reads and the step's barrier serve twice the MFMAs),
+// resident in registers as MFMA B operands.  It streams every unit of expanded rows that can see them: unit
 // (query block ib, delta) is the 32 rows r = (i0 + r, k = i - delta) with
 // Q~[r] = q[i] * k2~[k] * scale*log2(e) and dO~[r] = dO[i] * v2~[k], formed by the whole
 // workgroup into a three-deep LDS ring one step ahead of their use.  Per unit and pair:
@@ -12,6 +14,10 @@
 // Transposed operands come from the same unit tiles through ds_read_b64_tr_b16; the tiles are laid
 // out in row groups so that both kinds of read are free of bank conflicts.
 // Every output element has one writer and a fixed summation order.
+//
+// Small grids (fewer workgroups than the chip holds) split the stream of query blocks of a key block
+// over up to eight workgroups; each writes its fp32 partial dK and dV to the workspace and
+// kv_sum_kernel adds the partials in split order.
 #include <type_traits>
 
 #include "sa2_mfma_common.h"
@@ -22,10 +28,13 @@ namespace {
 constexpr int VW = 8;                  // wavefronts per workgroup
 constexpr int VT = VW * 64;            // threads per workgroup
 constexpr int VPAIR = 4;
-constexpr int VJ = VPAIR * 32;         // K rows per workgroup
+constexpr int KV_MAX_SPLIT = 8;        // workgroups a key block's query blocks are split over, at most
+constexpr int KV_GRID_TARGET = 512;    // a split stops once the grid holds this many workgroups
 
-template <int D>
+// KB: 32-row blocks of K/V rows per wavefront pair
+template <int D, int KB>
 struct KvCfg {
+    static constexpr int VJ = VPAIR * 32 * KB;     // K rows per workgroup
     static constexpr int DK = D / 16;
     static constexpr int DT = D / 32;
     // A unit tile (32 rows) in LDS keeps groups of RPW rows together: within a group the 16-byte
@@ -39,7 +48,7 @@ struct KvCfg {
     static constexpr int NUNIT = 3;
     static constexpr int RS = D + D / 4;       // K'/V' row stride (bf16): the forming threads' reads (RPW rows x 16 bytes per 16 lanes) hit distinct banks
     static constexpr int FS = D;               // q / dO row stride (fp32); read once per query block, unpadded
-    static constexpr int PX_BYTES = VPAIR * 2 * 64 * 32;
+    static constexpr int PX_BYTES = VPAIR * 2 * KB * 64 * 32;
     static constexpr size_t LDS_LIMIT = 160 * 1024;
     static size_t lds_bytes(int w2) {
         return (size_t)NUNIT * UNIT_BYTES + PX_BYTES + 2 * BQ * FS * 4 + 2 * (size_t)(BQ + w2) * RS * 2 + 4 * BQ * 4;
@@ -48,12 +57,15 @@ struct KvCfg {
 };
 
 // BIAS = false: k2_bias and v2_bias are both zero (the reference's default), the adds drop out.
-template <class E, int D, bool BIAS>
+// nsplit > 1: the workgroup takes the sp-th share of the key block's query blocks and writes fp32
+// partial sums to `part` ([2][nsplit][B*H][N][D]: dK before its scale, then dV).
+template <class E, int D, bool BIAS, int KB>
 __global__ __launch_bounds__(VT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
+void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __restrict__ part) {
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
-    using C = KvCfg<D>;
+    using C = KvCfg<D, KB>;
+    constexpr int VJ = C::VJ;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int SR = BQ + w2;                                   // K'/V' rows kept per query block
@@ -73,12 +85,11 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
 
     int pid = blockIdx.x;
     if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    const int bh = pid / njb, jb = pid - bh * njb;
+    const int sp = pid % nsplit, pj = pid / nsplit;
+    const int bh = pj / njb, jb = pj - bh * njb;
     const int b = bh / p.H, h = bh - b * p.H;
     const int j0 = jb * VJ;
-    const int jw = j0 + 32 * pr;                 // this pair's K rows: jw .. jw+31
-    const int j = jw + ln;
-    const int jc = j < N ? j : N - 1;
+    const int jw = j0 + 32 * KB * pr;            // this pair's K rows: jw .. jw+32*KB-1, in blocks of 32
 
     const uint16_t* qp = (const uint16_t*)p.q.p + p.q.off(b, 0, h);
     const uint16_t* k2p = (const uint16_t*)p.k2.p + p.k2.off(b, 0, h);
@@ -86,23 +97,34 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
 
     // K rows (P wavefront) or V rows (dS wavefront) of the pair as the resident B operand
-    X8 kvf[C::DK];
-    {
+    X8 kvf[KB][C::DK];
+#pragma unroll
+    for (int sb = 0; sb < KB; ++sb) {
         const Tensor& t = role ? p.v1 : p.k1;
-        const uint16_t* src = (const uint16_t*)t.p + t.off(b, jc, h) + hf * 8;
+        const int j = jw + 32 * sb + ln;
+        const uint16_t* src = (const uint16_t*)t.p + t.off(b, j < N ? j : N - 1, h) + hf * 8;
 #pragma unroll
-        for (int kk = 0; kk < C::DK; ++kk) kvf[kk] = *(const X8*)(src + kk * 16);
+        for (int kk = 0; kk < C::DK; ++kk) kvf[sb][kk] = *(const X8*)(src + kk * 16);
     }
-    floatx16 oacc[C::DT];                        // dV^T (P wavefront) or dK^T (dS wavefront)
+    floatx16 oacc[KB][C::DT];                    // dV^T (P wavefront) or dK^T (dS wavefront)
 #pragma unroll
-    for (int dt = 0; dt < C::DT; ++dt)
+    for (int sb = 0; sb < KB; ++sb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[dt][v] = 0.f;
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[sb][dt][v] = 0.f;
 
     const float qscale = p.scale * LOG2E;
     const int j_last = (j0 + VJ - 1 < N ? j0 + VJ - 1 : N - 1);
     const int i_max = (int)((int64_t)j_last + w1 < N - 1 ? j_last + w1 : N - 1);
-    const int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+    // the query blocks that see the key block, and this workgroup's share of them
+    int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+    if (nsplit > 1) {
+        const int chunk = (ib_hi - ib_lo + nsplit) / nsplit;
+        ib_lo += sp * chunk;
+        ib_hi = ib_hi < ib_lo + chunk - 1 ? ib_hi : ib_lo + chunk - 1;
+    }
+    const bool has_work = ib_lo <= ib_hi;
     auto units_of = [&](int ib) {
         const int il = (ib * BQ + BQ - 1 < N ? ib * BQ + BQ - 1 : N - 1);
         return (w2 < il ? w2 : il) + 1;
@@ -185,7 +207,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     };
 
     const uint32_t units_addr = lds_address(units);
-    const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * 64 * 32 + lane * 32);
+    const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * KB * 64 * 32 + lane * 32);
     // this lane's part of a row operand read (row ln, the k-slots of its half; k-step kk adds
     // kk * KKB) and of a transposed operand read (32-column block dt adds dt * DTB)
     const uint32_t row_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);
@@ -193,11 +215,13 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;
 
     // ---- prologue: first block's raw rows, first unit --------------------------------
-    load_raw(ib_lo);
-    __syncthreads();
-    fetch_qd();
-    form(0, 0);
-    __syncthreads();
+    if (has_work) {
+        load_raw(ib_lo);
+        __syncthreads();
+        fetch_qd();
+        form(0, 0);
+        __syncthreads();
+    }
 
     // The sweep, instantiated once per role so that each keeps only its own registers live.
     auto sweep = [&](auto role_tag) {
@@ -208,40 +232,60 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
         floatx16 negr;                               // -LSE*log2e (P) or -D (dS) of the block's rows, per accumulator element
     #pragma unroll
         for (int v = 0; v < 16; ++v) negr[v] = 0.f;
-        floatx16 dp_prev;
+        floatx16 dp_prev[KB];
     #pragma unroll
-        for (int v = 0; v < 16; ++v) dp_prev[v] = 0.f;
-        bool act_prev = false;
+        for (int sb = 0; sb < KB; ++sb)
+    #pragma unroll
+            for (int v = 0; v < 16; ++v) dp_prev[sb][v] = 0.f;
+        bool act_prev[KB];
+    #pragma unroll
+        for (int sb = 0; sb < KB; ++sb) act_prev[sb] = false;
 
         // dS of the previous unit and its dK MFMAs (dS wavefronts)
         auto consume = [&](int pslot, int pstep) {
             typedef const X8 __attribute__((address_space(3)))* lds_b8;
-            const uint32_t a = px_addr + (uint32_t)((pstep & 1) * 64 * 32);
-            const X8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
             const uint32_t qt_addr = units_addr + (uint32_t)(pslot * C::UNIT_BYTES) + col_lane;
             X8 qt[C::DT][2];
     #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
     #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) qt[dt][ks] = lds_group_column_operand_at<C, X8>(qt_addr + dt * DTB, ks);
-            X8 dsb[2];
     #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                dsb[0][t] = (EL)((float)p0[t] * dp_prev[t]);
-                dsb[1][t] = (EL)((float)p1[t] * dp_prev[8 + t]);
+            for (int sb = 0; sb < KB; ++sb) {
+                if (!act_prev[sb]) continue;
+                const uint32_t a = px_addr + (uint32_t)(((pstep & 1) * KB + sb) * 64 * 32);
+                const X8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
+                X8 dsb[2];
+    #pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    dsb[0][t] = (EL)((float)p0[t] * dp_prev[sb][t]);
+                    dsb[1][t] = (EL)((float)p1[t] * dp_prev[sb][8 + t]);
+                }
+    #pragma unroll
+                for (int dt = 0; dt < C::DT; ++dt)
+    #pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+                        oacc[sb][dt] = E::mfma(qt[dt][ks], dsb[ks], oacc[sb][dt], 0, 0, 0);
             }
+        };
+        auto any_of = [&](const bool (&x)[KB]) {
+            bool r = false;
     #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt)
-    #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
-                    oacc[dt] = E::mfma(qt[dt][ks], dsb[ks], oacc[dt], 0, 0, 0);
+            for (int sb = 0; sb < KB; ++sb) r |= x[sb];
+            return r;
         };
 
         while (true) {
             const int i0 = ib * BQ;
-            // does this pair's K tile see any query of the block?
-            const bool act = (i0 + BQ - 1 >= jw) && ((int64_t)i0 <= (int64_t)jw + 31 + w1) && jw < N;
-            if (act && cur_ib != ib) {
+            // which of this pair's K blocks see a query of the block?
+            bool act[KB];
+    #pragma unroll
+            for (int sb = 0; sb < KB; ++sb) {
+                const int jb0 = jw + 32 * sb;
+                act[sb] = (i0 + BQ - 1 >= jb0) && ((int64_t)i0 <= (int64_t)jb0 + 31 + w1) && jb0 < N;
+            }
+            const bool act_any = any_of(act);
+            if (act_any && cur_ib != ib) {
                 const float* src = (ROLE ? dsum_s : lse_s) + (ib & 1) * BQ + 4 * hf;
     #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
@@ -252,42 +296,47 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             }
             const uint32_t u_addr = units_addr + (uint32_t)(slot * C::UNIT_BYTES);
             if (ROLE == 0) {
-                if (act) {
+                if (act_any) {
                     X8 qa[C::DK];
     #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) qa[kk] = lds_read_x8<X8>(u_addr + row_lane + kk * KKB);
-                    floatx16 sh;
-                    const bool interior = (i0 >= jw + 31) && ((int64_t)i0 + 31 <= (int64_t)jw + w1) && (i0 + BQ - 1 < N) &&
-                                          (i0 >= delta);
-                    if (__builtin_expect(interior, 1)) {
-                        sh = E::mfma(qa[0], kvf[0], negr, 0, 0, 0);
-                    } else {
-                        asm volatile("" ::: "memory");
-                        // element v of this lane is query i0 + 8*(v/4) + 4*hf + v%4, column j
-                        const int lo = j - i0 - 4 * hf;
-                        const int hi = (int)((int64_t)j + w1 - i0 < 1 << 20 ? j + w1 - i0 : 1 << 20) - 4 * hf;
-                        const int dlo = delta - i0 - 4 * hf, nhi = N - 1 - i0 - 4 * hf;
-                        floatx16 ct;
+                    X8 pb[KB][2];
     #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int c = 8 * (v >> 2) + (v & 3);
-                            ct[v] = ((j < N) & (c >= lo) & (c <= hi) & (c >= dlo) & (c <= nhi)) ? negr[v] : -INFINITY;
+                    for (int sb = 0; sb < KB; ++sb) {
+                        if (!act[sb]) continue;
+                        const int jb0 = jw + 32 * sb, j = jb0 + ln;
+                        floatx16 sh;
+                        const bool interior = (i0 >= jb0 + 31) && ((int64_t)i0 + 31 <= (int64_t)jb0 + w1) && (i0 + BQ - 1 < N) &&
+                                              (i0 >= delta);
+                        if (__builtin_expect(interior, 1)) {
+                            sh = E::mfma(qa[0], kvf[sb][0], negr, 0, 0, 0);
+                        } else {
+                            asm volatile("" ::: "memory");
+                            // element v of this lane is query i0 + 8*(v/4) + 4*hf + v%4, column j
+                            const int lo = j - i0 - 4 * hf;
+                            const int hi = (int)((int64_t)j + w1 - i0 < 1 << 20 ? j + w1 - i0 : 1 << 20) - 4 * hf;
+                            const int dlo = delta - i0 - 4 * hf, nhi = N - 1 - i0 - 4 * hf;
+                            floatx16 ct;
+    #pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                const int c = 8 * (v >> 2) + (v & 3);
+                                ct[v] = ((j < N) & (c >= lo) & (c <= hi) & (c >= dlo) & (c <= nhi)) ? negr[v] : -INFINITY;
+                            }
+                            sh = E::mfma(qa[0], kvf[sb][0], ct, 0, 0, 0);
                         }
-                        sh = E::mfma(qa[0], kvf[0], ct, 0, 0, 0);
-                    }
     #pragma unroll
-                    for (int kk = 1; kk < C::DK; ++kk)
-                        sh = E::mfma(qa[kk], kvf[kk], sh, 0, 0, 0);
-                    X8 pb[2];
+                        for (int kk = 1; kk < C::DK; ++kk)
+                            sh = E::mfma(qa[kk], kvf[sb][kk], sh, 0, 0, 0);
     #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
+                        for (int ks = 0; ks < 2; ++ks)
     #pragma unroll
-                        for (int t = 0; t < 8; ++t) pb[ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
-                    {
-                        typedef X8 __attribute__((address_space(3)))* lds_b8;
-                        const uint32_t a = px_addr + (uint32_t)((step & 1) * 64 * 32);
-                        *(lds_b8)(uintptr_t)a = pb[0];
-                        *(lds_b8)(uintptr_t)(a + 16) = pb[1];
+                            for (int t = 0; t < 8; ++t) pb[sb][ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
+                        {
+                            typedef X8 __attribute__((address_space(3)))* lds_b8;
+                            const uint32_t a = px_addr + (uint32_t)(((step & 1) * KB + sb) * 64 * 32);
+                            *(lds_b8)(uintptr_t)a = pb[sb][0];
+                            *(lds_b8)(uintptr_t)(a + 16) = pb[sb][1];
+                        }
                     }
                     const uint32_t dt_addr = u_addr + (uint32_t)C::TILE_BYTES + col_lane;
                     X8 da[C::DT][2];
@@ -296,27 +345,38 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
     #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) da[dt][ks] = lds_group_column_operand_at<C, X8>(dt_addr + dt * DTB, ks);
     #pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
+                    for (int sb = 0; sb < KB; ++sb) {
+                        if (!act[sb]) continue;
     #pragma unroll
-                        for (int ks = 0; ks < 2; ++ks)
-                            oacc[dt] = E::mfma(da[dt][ks], pb[ks], oacc[dt], 0, 0, 0);
+                        for (int dt = 0; dt < C::DT; ++dt)
+    #pragma unroll
+                            for (int ks = 0; ks < 2; ++ks)
+                                oacc[sb][dt] = E::mfma(da[dt][ks], pb[sb][ks], oacc[sb][dt], 0, 0, 0);
+                    }
                 }
             } else {
                 // first the previous unit (its dP is still in dp_prev), then this unit's dP
-                if (act_prev) consume(slot == 0 ? C::NUNIT - 1 : slot - 1, step - 1);
-                if (act) {
+                if (any_of(act_prev)) consume(slot == 0 ? C::NUNIT - 1 : slot - 1, step - 1);
+                if (act_any) {
                     const uint32_t d_addr = u_addr + (uint32_t)C::TILE_BYTES;
                     X8 da[C::DK];
     #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) da[kk] = lds_read_x8<X8>(d_addr + row_lane + kk * KKB);
-                    dp_prev = E::mfma(da[0], kvf[0], negr, 0, 0, 0);
     #pragma unroll
-                    for (int kk = 1; kk < C::DK; ++kk)
-                        dp_prev = E::mfma(da[kk], kvf[kk], dp_prev, 0, 0, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
+                    for (int sb = 0; sb < KB; ++sb) {
+                        if (!act[sb]) continue;
+                        dp_prev[sb] = E::mfma(da[0], kvf[sb][0], negr, 0, 0, 0);
+    #pragma unroll
+                        for (int kk = 1; kk < C::DK; ++kk)
+                            dp_prev[sb] = E::mfma(da[kk], kvf[sb][kk], dp_prev[sb], 0, 0, 0);
+                    }
+                    if constexpr (KB == 1) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
+                    }
                 }
-                act_prev = act;
+    #pragma unroll
+                for (int sb = 0; sb < KB; ++sb) act_prev[sb] = act[sb];
             }
 
             // ---- next unit: form it one step ahead (after a change of block: its raw rows first)
@@ -344,49 +404,138 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total) {
             delta = ndelta;
             slot = nslot;
         }
-        if (ROLE == 1 && act_prev) consume(slot, step - 1);
+        if (ROLE == 1 && any_of(act_prev)) consume(slot, step - 1);
 
     };
-    if (role == 0) sweep(std::integral_constant<int, 0>());
-    else sweep(std::integral_constant<int, 1>());
+    if (has_work) {
+        if (role == 0) sweep(std::integral_constant<int, 0>());
+        else sweep(std::integral_constant<int, 1>());
+    }
 
-    if (j < N) {
-        const Tensor& t = role ? p.dk1 : p.dv1;
-        if (t.p) {
+    const Tensor& t = role ? p.dk1 : p.dv1;
+    const float sc = role ? LN2 : 1.f;               // Q~ carries scale*log2(e)
+#pragma unroll
+    for (int sb = 0; sb < KB; ++sb) {
+        const int j = jw + 32 * sb + ln;
+        if (j >= N || !t.p) continue;
+        if (nsplit == 1) {
             uint16_t* dst = (uint16_t*)t.p + t.off(b, j, h) + 4 * hf;
-            const float sc = role ? LN2 : 1.f;       // Q~ carries scale*log2(e)
 #pragma unroll
             for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     union { EL hh[4]; uint2 u; } a;
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) a.hh[x] = (EL)(oacc[dt][4 * g4 + x] * sc);
+                    for (int x = 0; x < 4; ++x) a.hh[x] = (EL)(oacc[sb][dt][4 * g4 + x] * sc);
                     *(uint2*)(dst + dt * 32 + 8 * g4) = a.u;
                 }
+        } else {
+            // fp32 partial of this share: [dK | dV][split][batch*head][position][column]
+            const int64_t BH = (int64_t)p.B * p.H;
+            float* dst = part + ((((role ? 0 : 1) * (int64_t)nsplit + sp) * BH + bh) * N + j) * D + 4 * hf;
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4)
+                    *(float4*)(dst + dt * 32 + 8 * g4) = make_float4(oacc[sb][dt][4 * g4] * sc, oacc[sb][dt][4 * g4 + 1] * sc,
+                                                                     oacc[sb][dt][4 * g4 + 2] * sc, oacc[sb][dt][4 * g4 + 3] * sc);
         }
     }
 }
 
-template <class E, int D>
-int launch_kv(const Problem& p, hipStream_t st) {
-    using C = KvCfg<D>;
-    const int njb = (p.N + VJ - 1) / VJ;
-    const int64_t total = (int64_t)njb * p.B * p.H;
+// dK and dV from the partial sums of a split launch, shares added in their order
+template <class E>
+__global__ __launch_bounds__(256) void kv_sum_kernel(Problem p, int nsplit, const float* __restrict__ part, int64_t chunks) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= chunks) return;
+    const int D = p.D;
+    const int col = (int)(c % (D / 4));
+    const int64_t rowid = c / (D / 4);
+    const int j = (int)(rowid % p.N);
+    const int bh = (int)(rowid / p.N);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int64_t BH = (int64_t)p.B * p.H;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const Tensor& t = which ? p.dv1 : p.dk1;
+        if (!t.p) continue;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < nsplit; ++s) {
+            const float4 y = *(const float4*)(part + (((which * (int64_t)nsplit + s) * BH + bh) * p.N + j) * D + col * 4);
+            acc.x += y.x; acc.y += y.y; acc.z += y.z; acc.w += y.w;
+        }
+        *(uint2*)((uint16_t*)t.p + t.off(b, j, h) + col * 4) = make_uint2(E::pack(acc.x, acc.y), E::pack(acc.z, acc.w));
+    }
+}
+
+// Geometry of a launch: 32-row K blocks per wavefront pair, and the number of shares a key block's
+// query blocks are split into.  Both depend on the problem's sizes only.
+struct KvPlan {
+    int kb, nsplit;
+};
+KvPlan kv_plan(int B, int N, int H, int D, int w1) {
+    KvPlan pl{1, 1};
+    const int64_t bh = (int64_t)B * H;
+    // two K blocks per pair at head_dim 64 when that still leaves a grid worth splitting no further than in two
+    if (D == 64 && bh * ((N + 255) / 256) * 2 >= KV_GRID_TARGET / 2) pl.kb = 2;
+    const int vj = VPAIR * 32 * pl.kb;
+    const int64_t base = bh * ((N + vj - 1) / vj);
+    const int blocks = (vj + (w1 < N ? w1 : N) + BQ - 1) / BQ + 1;          // query blocks a key block streams, at most
+    // (the partial sums of a split launch stay under 32 MiB)
+    auto part_bytes = [&](int ns) { return (int64_t)2 * ns * bh * N * D * 4; };
+    while (pl.nsplit < KV_MAX_SPLIT && base * pl.nsplit * 2 <= KV_GRID_TARGET && pl.nsplit * 2 <= blocks &&
+           part_bytes(pl.nsplit * 2) <= ((int64_t)32 << 20))
+        pl.nsplit *= 2;
+    return pl;
+}
+
+template <class E, int D, int KB>
+int launch_kv_geometry(const Problem& p, int nsplit, hipStream_t st) {
+    using C = KvCfg<D, KB>;
+    const int njb = (p.N + C::VJ - 1) / C::VJ;
+    const int64_t total = (int64_t)njb * p.B * p.H * nsplit;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
     const size_t lds = C::lds_bytes(p.w2);
     const bool bias = p.k2_bias != 0.f || p.v2_bias != 0.f;
-    const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<E, D, true> : (const void*)mfma_bwd_kv_kernel<E, D, false>;
+    // the partial sums of a split launch lie behind the K'-side kernel's part of the workspace
+    float* part = nullptr;
+    if (nsplit > 1) {
+        const size_t off = kp_side_scratch_bytes(p.B, p.N, p.H, D, p.w2);
+        if (p.scratch_bytes < off + kv_split_scratch_bytes(p.B, p.N, p.H, D, p.w1)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+        part = (float*)((char*)p.scratch + off);
+    }
+    const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<E, D, true, KB> : (const void*)mfma_bwd_kv_kernel<E, D, false, KB>;
     if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
-    if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
-    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total);
-    return hipGetLastError() == hipSuccess ? SA2_OK : SA2_ERR_LAUNCH_FAILED;
+    if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true, KB>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part);
+    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false, KB>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part);
+    if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    if (nsplit > 1) {
+        const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
+        hipLaunchKernelGGL((kv_sum_kernel<E>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, p, nsplit, part, chunks);
+        if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    }
+    return SA2_OK;
+}
+
+template <class E, int D>
+int launch_kv(const Problem& p, hipStream_t st) {
+    const KvPlan pl = kv_plan(p.B, p.N, p.H, D, p.w1);
+    if constexpr (D == 64) {
+        if (pl.kb == 2) return launch_kv_geometry<E, D, 2>(p, pl.nsplit, st);
+    }
+    return launch_kv_geometry<E, D, 1>(p, pl.nsplit, st);
 }
 
 }  // namespace
 
 bool kv_fits(int D, int w2) {
-    return D == 128 ? KvCfg<128>::fits(w2) : D == 64 ? KvCfg<64>::fits(w2) : D == 32 ? KvCfg<32>::fits(w2) : false;
+    // (two K blocks per pair need the larger hand-over buffer: the limit is theirs at head_dim 64)
+    return D == 128 ? KvCfg<128, 1>::fits(w2) : D == 64 ? KvCfg<64, 2>::fits(w2) : D == 32 ? KvCfg<32, 1>::fits(w2) : false;
+}
+
+size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1) {
+    const KvPlan pl = kv_plan(B, N, H, D, w1);
+    return pl.nsplit > 1 ? (size_t)2 * pl.nsplit * B * H * (size_t)N * D * sizeof(float) : 0;
 }
 
 int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st) {

@@ -35,6 +35,11 @@ def _both_backwards(shape, w, dtype, seed, flags, inclusive=1, needs=(True,) * 5
         head += [g.data_ptr() if need else None for g, need in zip(grads, needs)]      # NULL = not needed
         tail = [B, N, H, D, strides, w[0], w[1], scale, 0.0, 0.0, DT[dtype], inclusive, flags, stream]
         if static:
+            # The first call on a device looks up the library's array (the runtime places it in device
+            # memory then) and sets kernel attributes; every later call only launches kernels.
+            _lib.check(lib.sa2_backward_static_workspace(*head, *tail))
+            for g in grads:
+                g.fill_(7.0)
             torch.cuda.synchronize()
             free_before = torch.cuda.mem_get_info(dev)[0]
             _lib.check(lib.sa2_backward_static_workspace(*head, *tail))
