@@ -191,11 +191,11 @@ size_t sa2_bwd_workspace_bytes(int B, int N, int H, int D, int w1, int w2, int d
         if (m > scratch) scratch = m;
     }
     if (!(flags & SA2_FLAG_FORCE_GENERIC) && wide_bwd_supported(D, reach(w2, 1, N), dtype)) {
-        const size_t m = wide_bwd_scratch_bytes(B, N, H, D, reach(w2, 1, N));
+        const size_t m = wide_bwd_scratch_bytes(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N));
         if (m > scratch) scratch = m;
     }
     if (!(flags & SA2_FLAG_FORCE_GENERIC) && f32_mfma_bwd_supported(D, reach(w2, 1, N), dtype)) {
-        const size_t m = f32_mfma_bwd_scratch_bytes(B, N, H, D, reach(w2, 1, N));
+        const size_t m = f32_mfma_bwd_scratch_bytes(B, N, H, D, reach(w1, 1, N), reach(w2, 1, N));
         if (m > scratch) scratch = m;
     }
     return dsum_bytes(B, N, H) + align_up(scratch, 256) + 256;

@@ -89,13 +89,13 @@ size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 bool f32_mfma_supported(int D, int dtype);
 bool f32_mfma_bwd_supported(int D, int w2, int dtype);
 bool f32_mfma_layout_ok(const Problem& p, bool backward);
-size_t f32_mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w2);
+size_t f32_mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 int launch_f32_mfma_fwd(const Problem& p, hipStream_t st);
 int launch_f32_mfma_bwd(const Problem& p, hipStream_t st);
 // 16-bit tensors with head_dim 256 on the 16-bit MFMA (rows 16-byte aligned)
 bool wide_supported(int D, int dtype);
 bool wide_bwd_supported(int D, int w2, int dtype);
-size_t wide_bwd_scratch_bytes(int B, int N, int H, int D, int w2);
+size_t wide_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 int launch_wide_fwd(const Problem& p, int dtype, hipStream_t st);
 int launch_wide_bwd(const Problem& p, int dtype, hipStream_t st);
 // K'-side backward kernel (dQ, dK', dV') that keeps its partial sums on chip

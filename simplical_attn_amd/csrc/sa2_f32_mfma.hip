@@ -515,9 +515,12 @@ __global__ __launch_bounds__(256) void f32_dq_sum_kernel(Problem p, int nkb, con
 }
 
 // =================================================== backward, K side: dK, dV =====
-template <int D>
+// nsplit > 1 (grids smaller than the chip): the workgroup takes the sp-th share of the key block's query
+// blocks and writes fp32 partial sums to `part` ([dK | dV][nsplit][B*H][N][D]) for f32_kv_sum_kernel.
+template <int D, bool SPLIT>
 __global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void f32_bwd_kv_kernel(Problem p, int njb, int total) {
+void f32_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __restrict__ part) {
+    const int nsplit = SPLIT ? nsplit_arg : 1;
     using C = F32Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) float smem_f[];
     float* lse_s = smem_f + 2 * C::STAGE;        // [2][32]  LSE*log2(e) of the unit's queries
@@ -527,7 +530,8 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, ln = lane & 31, hf = lane >> 5;
     const int pid = xcd_order(blockIdx.x, total);
-    const int bh = pid / njb, jb = pid - bh * njb;
+    const int sp = pid % nsplit, pj = pid / nsplit;
+    const int bh = pj / njb, jb = pj - bh * njb;
     const int b = bh / p.H, h = bh - b * p.H;
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int j0 = jb * XJ, jw = j0 + 32 * wave, j = jw + ln, jc = j < N ? j : N - 1;
@@ -555,7 +559,16 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total) {
 
     const int j_last = j0 + XJ - 1 < N ? j0 + XJ - 1 : N - 1;
     const int i_max = (int)((int64_t)j_last + w1 < N - 1 ? j_last + w1 : N - 1);
-    const int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+    // the query blocks that see the key block, and this workgroup's share of them
+    int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+    if constexpr (SPLIT) {
+        const int chunk = (ib_hi - ib_lo + nsplit) / nsplit;
+        ib_lo += sp * chunk;
+        ib_hi = ib_hi < ib_lo + chunk - 1 ? ib_hi : ib_lo + chunk - 1;
+    }
+    // (a share of a split launch may be empty: it walks one block without touching it and writes zeros)
+    const bool empty_share = ib_lo > ib_hi;
+    if (empty_share) ib_lo = ib_hi = j0 / BQ;
     auto units_of = [&](int ib) {
         const int il = ib * BQ + BQ - 1 < N ? ib * BQ + BQ - 1 : N - 1;
         return (w2 < il ? w2 : il) + 1;
@@ -617,7 +630,7 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total) {
         if (more) fetch_unit(nib, ndelta);
 
         const int i0 = ib * BQ;
-        const bool touches = (i0 + BQ - 1 >= jw) && ((int64_t)i0 <= (int64_t)jw + 31 + w1) && jw < N;
+        const bool touches = (i0 + BQ - 1 >= jw) && ((int64_t)i0 <= (int64_t)jw + 31 + w1) && jw < N && !empty_share;
         if (touches) {
             const float* Qs = smem_f + buf * C::STAGE;
             const float* Ds = Qs + C::TILE;
@@ -676,6 +689,11 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total) {
     if (j < N) {
         float* dkp = p.dk1.p ? (float*)p.dk1.p + p.dk1.off(b, j, h) + 4 * hf : nullptr;
         float* dvp = p.dv1.p ? (float*)p.dv1.p + p.dv1.off(b, j, h) + 4 * hf : nullptr;
+        if constexpr (SPLIT) {
+            const int64_t BH = (int64_t)p.B * p.H;
+            if (dkp) dkp = part + (((0 * (int64_t)nsplit + sp) * BH + bh) * N + j) * D + 4 * hf;
+            if (dvp) dvp = part + (((1 * (int64_t)nsplit + sp) * BH + bh) * N + j) * D + 4 * hf;
+        }
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -687,6 +705,42 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total) {
                                                                            dvacc[dt][4 * g4 + 3]);
             }
     }
+}
+
+// dK and dV from the partial sums of a split launch, shares added in their order
+template <int D>
+__global__ __launch_bounds__(256) void f32_kv_sum_kernel(Problem p, int nsplit, const float* __restrict__ part, int64_t chunks) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= chunks) return;
+    const int col = (int)(c % (D / 4));
+    const int64_t rowid = c / (D / 4);
+    const int j = (int)(rowid % p.N);
+    const int bh = (int)(rowid / p.N);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int64_t BH = (int64_t)p.B * p.H;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const Tensor& t = which ? p.dv1 : p.dk1;
+        if (!t.p) continue;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < nsplit; ++s) {
+            const float4 y = *(const float4*)(part + (((which * (int64_t)nsplit + s) * BH + bh) * p.N + j) * D + col * 4);
+            acc.x += y.x; acc.y += y.y; acc.z += y.z; acc.w += y.w;
+        }
+        *(float4*)((float*)t.p + t.off(b, j, h) + col * 4) = acc;
+    }
+}
+
+// Shares a key block's query blocks are split into when the K-side grid is smaller than the chip
+int f32_kv_nsplit(int B, int N, int H, int D, int w1) {
+    const int64_t bh = (int64_t)B * H, base = bh * ((N + XJ - 1) / XJ);
+    const int blocks = (XJ + (w1 < N ? w1 : N) + BQ - 1) / BQ + 1;
+    int ns = 1;
+    while (ns < 8 && base * ns * 2 <= 512 && ns * 2 <= blocks && (int64_t)2 * ns * 2 * bh * N * D * 4 <= ((int64_t)32 << 20)) ns *= 2;
+    return ns;
+}
+size_t f32_dq_part_bytes(int B, int N, int H, int D, int w2) {
+    return ((size_t)B * H * ((N + BQ - 1) / BQ) * (size_t)(32 + w2) * D * sizeof(float) + 255) / 256 * 256;
 }
 
 // ------------------------------------------------------------------ launchers ----
@@ -710,7 +764,7 @@ int launch_f32_bwd(const Problem& p, hipStream_t st) {
         const int nkb = (p.N + BQ - 1) / BQ;
         const int64_t total = (int64_t)nkb * p.B * p.H;
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-        if (p.scratch_bytes < f32_mfma_bwd_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+        if (p.scratch_bytes < f32_dq_part_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
         float* part = (float*)p.scratch;
         if (!allow_full_lds((const void*)f32_bwd_kp_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
         hipLaunchKernelGGL((f32_bwd_kp_kernel<D>), dim3((unsigned)total), dim3(XT), C::kp_lds(p.w2), st, p, nkb, (int)total, part);
@@ -723,11 +777,26 @@ int launch_f32_bwd(const Problem& p, hipStream_t st) {
     }
     if (p.dk1.p || p.dv1.p) {
         const int njb = (p.N + XJ - 1) / XJ;
-        const int64_t total = (int64_t)njb * p.B * p.H;
+        const int nsplit = f32_kv_nsplit(p.B, p.N, p.H, D, p.w1);
+        const int64_t total = (int64_t)njb * p.B * p.H * nsplit;
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-        if (!allow_full_lds((const void*)f32_bwd_kv_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL((f32_bwd_kv_kernel<D>), dim3((unsigned)total), dim3(XT), C::KV_LDS, st, p, njb, (int)total);
+        float* kv_part = nullptr;
+        if (nsplit > 1) {
+            if (p.scratch_bytes < f32_mfma_bwd_scratch_bytes(p.B, p.N, p.H, D, p.w1, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+            kv_part = (float*)((char*)p.scratch + f32_dq_part_bytes(p.B, p.N, p.H, D, p.w2));
+        }
+        if (!allow_full_lds((const void*)f32_bwd_kv_kernel<D, false>) || !allow_full_lds((const void*)f32_bwd_kv_kernel<D, true>))
+            return SA2_ERR_LAUNCH_FAILED;
+        if (nsplit > 1)
+            hipLaunchKernelGGL((f32_bwd_kv_kernel<D, true>), dim3((unsigned)total), dim3(XT), C::KV_LDS, st, p, njb, (int)total, nsplit, kv_part);
+        else
+            hipLaunchKernelGGL((f32_bwd_kv_kernel<D, false>), dim3((unsigned)total), dim3(XT), C::KV_LDS, st, p, njb, (int)total, 1, kv_part);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+        if (nsplit > 1) {
+            const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
+            hipLaunchKernelGGL((f32_kv_sum_kernel<D>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, p, nsplit, kv_part, chunks);
+            if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+        }
     }
     return SA2_OK;
 }
@@ -759,8 +828,9 @@ bool f32_mfma_layout_ok(const Problem& p, bool backward) {
     return true;
 }
 
-size_t f32_mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w2) {
-    return (size_t)B * H * ((N + BQ - 1) / BQ) * (size_t)(32 + w2) * D * sizeof(float);
+size_t f32_mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
+    const int ns = f32_kv_nsplit(B, N, H, D, w1);
+    return f32_dq_part_bytes(B, N, H, D, w2) + (ns > 1 ? (size_t)2 * ns * B * H * (size_t)N * D * sizeof(float) : 0);
 }
 
 int launch_f32_mfma_fwd(const Problem& p, hipStream_t st) {

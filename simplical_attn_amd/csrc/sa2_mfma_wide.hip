@@ -549,9 +549,12 @@ __global__ __launch_bounds__(256) void wide_dq_sum_kernel(Problem p, int nkb, co
 }
 
 // =================================================== backward, K side: dK, dV =====
-template <class E, int D, int DV>
+// nsplit > 1 (grids smaller than the chip): the workgroup takes the sp-th share of the key block's query
+// blocks and writes fp32 partial sums to `part` ([dK | dV][nsplit][B*H][N][D]) for wide_kv_sum_kernel.
+template <class E, int D, int DV, bool SPLIT>
 __global__ __launch_bounds__(WT) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void wide_kv_kernel(Problem p, int njb, int total) {
+void wide_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __restrict__ part) {
+    const int nsplit = SPLIT ? nsplit_arg : 1;
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
     using C = WideCfg<D, DV>;
@@ -565,7 +568,8 @@ void wide_kv_kernel(Problem p, int njb, int total) {
     const int lane = tid & 63, ln = lane & 31, hf = lane >> 5;
     const int pid = xcd_neighbours(blockIdx.x, total);
     const int c0 = blockIdx.y * DV;
-    const int bh = pid / njb, jb = pid - bh * njb;
+    const int sp = pid % nsplit, pj = pid / nsplit;
+    const int bh = pj / njb, jb = pj - bh * njb;
     const int b = bh / p.H, h = bh - b * p.H;
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int j0 = jb * WJ, jw = j0 + 32 * wave, j = jw + ln, jc = j < N ? j : N - 1;
@@ -593,7 +597,16 @@ void wide_kv_kernel(Problem p, int njb, int total) {
 
     const int j_last = j0 + WJ - 1 < N ? j0 + WJ - 1 : N - 1;
     const int i_max = (int)((int64_t)j_last + w1 < N - 1 ? j_last + w1 : N - 1);
-    const int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+    // the query blocks that see the key block, and this workgroup's share of them
+    int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
+    if constexpr (SPLIT) {
+        const int chunk = (ib_hi - ib_lo + nsplit) / nsplit;
+        ib_lo += sp * chunk;
+        ib_hi = ib_hi < ib_lo + chunk - 1 ? ib_hi : ib_lo + chunk - 1;
+    }
+    // (a share of a split launch may be empty: it walks one block without touching it and writes zeros)
+    const bool empty_share = ib_lo > ib_hi;
+    if (empty_share) ib_lo = ib_hi = j0 / BQ;
     auto units_of = [&](int ib) {
         const int il = ib * BQ + BQ - 1 < N ? ib * BQ + BQ - 1 : N - 1;
         return (w2 < il ? w2 : il) + 1;
@@ -652,7 +665,7 @@ void wide_kv_kernel(Problem p, int njb, int total) {
         if (more) fetch_unit(nib, ndelta);
 
         const int i0 = ib * BQ;
-        const bool touches = (i0 + BQ - 1 >= jw) && ((int64_t)i0 <= (int64_t)jw + 31 + w1) && jw < N;
+        const bool touches = (i0 + BQ - 1 >= jw) && ((int64_t)i0 <= (int64_t)jw + 31 + w1) && jw < N && !empty_share;
         if (touches) {
             const uint16_t* Qs = tiles + buf * C::STAGE;
             const uint16_t* Ds = Qs + C::TILE;
@@ -704,7 +717,20 @@ void wide_kv_kernel(Problem p, int njb, int total) {
         buf ^= 1;
     }
 
-    if (j < N) {
+    if (j < N && SPLIT) {
+        const int64_t BH = (int64_t)p.B * p.H;
+        float* dkp = p.dk1.p ? part + (((0 * (int64_t)nsplit + sp) * BH + bh) * N + j) * D + c0 + 4 * hf : nullptr;
+        float* dvp = p.dv1.p ? part + (((1 * (int64_t)nsplit + sp) * BH + bh) * N + j) * D + c0 + 4 * hf : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                if (dkp) *(float4*)(dkp + dt * 32 + 8 * g4) = make_float4(dkacc[dt][4 * g4] * LN2, dkacc[dt][4 * g4 + 1] * LN2,
+                                                                           dkacc[dt][4 * g4 + 2] * LN2, dkacc[dt][4 * g4 + 3] * LN2);
+                if (dvp) *(float4*)(dvp + dt * 32 + 8 * g4) = make_float4(dvacc[dt][4 * g4], dvacc[dt][4 * g4 + 1], dvacc[dt][4 * g4 + 2],
+                                                                           dvacc[dt][4 * g4 + 3]);
+            }
+    } else if (j < N) {
         uint16_t* dkp = p.dk1.p ? (uint16_t*)p.dk1.p + p.dk1.off(b, j, h) + c0 + 4 * hf : nullptr;
         uint16_t* dvp = p.dv1.p ? (uint16_t*)p.dv1.p + p.dv1.off(b, j, h) + c0 + 4 * hf : nullptr;
 #pragma unroll
@@ -718,6 +744,42 @@ void wide_kv_kernel(Problem p, int njb, int total) {
                                                                          E::pack(dvacc[dt][4 * g4 + 2], dvacc[dt][4 * g4 + 3]));
             }
     }
+}
+
+// dK and dV from the partial sums of a split launch, shares added in their order
+template <class E, int D>
+__global__ __launch_bounds__(256) void wide_kv_sum_kernel(Problem p, int nsplit, const float* __restrict__ part, int64_t chunks) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= chunks) return;
+    const int col = (int)(c % (D / 4));
+    const int64_t rowid = c / (D / 4);
+    const int j = (int)(rowid % p.N);
+    const int bh = (int)(rowid / p.N);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int64_t BH = (int64_t)p.B * p.H;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const Tensor& t = which ? p.dv1 : p.dk1;
+        if (!t.p) continue;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < nsplit; ++s) {
+            const float4 y = *(const float4*)(part + (((which * (int64_t)nsplit + s) * BH + bh) * p.N + j) * D + col * 4);
+            acc.x += y.x; acc.y += y.y; acc.z += y.z; acc.w += y.w;
+        }
+        *(uint2*)((uint16_t*)t.p + t.off(b, j, h) + col * 4) = make_uint2(E::pack(acc.x, acc.y), E::pack(acc.z, acc.w));
+    }
+}
+
+// Shares a key block's query blocks are split into when the K-side grid is smaller than the chip
+int wide_kv_nsplit(int B, int N, int H, int D, int w1, int npass) {
+    const int64_t bh = (int64_t)B * H, base = bh * ((N + WJ - 1) / WJ) * npass;
+    const int blocks = (WJ + (w1 < N ? w1 : N) + BQ - 1) / BQ + 1;
+    int ns = 1;
+    while (ns < 8 && base * ns * 2 <= 512 && ns * 2 <= blocks && (int64_t)2 * ns * 2 * bh * N * D * 4 <= ((int64_t)32 << 20)) ns *= 2;
+    return ns;
+}
+size_t wide_dq_part_bytes(int B, int N, int H, int D, int w2) {
+    return ((size_t)B * H * ((N + BQ - 1) / BQ) * (size_t)(32 + w2) * D * sizeof(float) + 255) / 256 * 256;
 }
 
 // ------------------------------------------------------------------ launchers ----
@@ -741,7 +803,7 @@ int launch_wide_bwd(const Problem& p, hipStream_t st) {
         const int nkb = (p.N + BQ - 1) / BQ;
         const int64_t total = (int64_t)nkb * p.B * p.H;
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-        if (p.scratch_bytes < wide_bwd_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+        if (p.scratch_bytes < wide_dq_part_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
         float* part = (float*)p.scratch;
         if (!allow_full_lds((const void*)wide_kp_kernel<E, D, DV>)) return SA2_ERR_LAUNCH_FAILED;
         hipLaunchKernelGGL((wide_kp_kernel<E, D, DV>), dim3((unsigned)total, C::NPASS), dim3(WT), C::kp_lds(p.w2), st, p, nkb, (int)total,
@@ -755,11 +817,28 @@ int launch_wide_bwd(const Problem& p, hipStream_t st) {
     }
     if (p.dk1.p || p.dv1.p) {
         const int njb = (p.N + WJ - 1) / WJ;
-        const int64_t total = (int64_t)njb * p.B * p.H;
+        const int nsplit = wide_kv_nsplit(p.B, p.N, p.H, D, p.w1, C::NPASS);
+        const int64_t total = (int64_t)njb * p.B * p.H * nsplit;
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-        if (!allow_full_lds((const void*)wide_kv_kernel<E, D, DV>)) return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL((wide_kv_kernel<E, D, DV>), dim3((unsigned)total, C::NPASS), dim3(WT), C::KV_LDS, st, p, njb, (int)total);
+        float* kv_part = nullptr;
+        if (nsplit > 1) {
+            if (p.scratch_bytes < wide_bwd_scratch_bytes(p.B, p.N, p.H, D, p.w1, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+            kv_part = (float*)((char*)p.scratch + wide_dq_part_bytes(p.B, p.N, p.H, D, p.w2));
+        }
+        if (!allow_full_lds((const void*)wide_kv_kernel<E, D, DV, false>) || !allow_full_lds((const void*)wide_kv_kernel<E, D, DV, true>))
+            return SA2_ERR_LAUNCH_FAILED;
+        if (nsplit > 1)
+            hipLaunchKernelGGL((wide_kv_kernel<E, D, DV, true>), dim3((unsigned)total, C::NPASS), dim3(WT), C::KV_LDS, st, p, njb, (int)total,
+                               nsplit, kv_part);
+        else
+            hipLaunchKernelGGL((wide_kv_kernel<E, D, DV, false>), dim3((unsigned)total, C::NPASS), dim3(WT), C::KV_LDS, st, p, njb, (int)total,
+                               1, kv_part);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+        if (nsplit > 1) {
+            const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
+            hipLaunchKernelGGL((wide_kv_sum_kernel<E, D>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, p, nsplit, kv_part, chunks);
+            if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+        }
     }
     return SA2_OK;
 }
@@ -770,8 +849,9 @@ bool wide_supported(int D, int dtype) { return (dtype == SA2_BF16 || dtype == SA
 
 bool wide_bwd_supported(int D, int w2, int dtype) { return wide_supported(D, dtype) && WideCfg<256, 128>::kp_fits(w2); }
 
-size_t wide_bwd_scratch_bytes(int B, int N, int H, int D, int w2) {
-    return (size_t)B * H * ((N + BQ - 1) / BQ) * (size_t)(32 + w2) * D * sizeof(float);
+size_t wide_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
+    const int ns = wide_kv_nsplit(B, N, H, D, w1, 2);
+    return wide_dq_part_bytes(B, N, H, D, w2) + (ns > 1 ? (size_t)2 * ns * B * H * (size_t)N * D * sizeof(float) : 0);
 }
 
 int launch_wide_fwd(const Problem& p, int dtype, hipStream_t st) {
