@@ -48,10 +48,11 @@ typedef enum sa2_status {
 typedef enum sa2_dtype { SA2_F32 = 0, SA2_BF16 = 1, SA2_F16 = 2 } sa2_dtype;
 
 /* flags */
-#define SA2_FLAG_AUTO 0u            /* MFMA kernels when the shape allows, generic otherwise */
+#define SA2_FLAG_AUTO 0u            /* matrix-pipe (MFMA) kernels when the shape allows, fp32-FMA kernels otherwise */
 #define SA2_FLAG_FORCE_GENERIC 1u   /* fp32-FMA kernels (any dtype, any D <= 256) */
-#define SA2_FLAG_FORCE_MFMA 2u      /* MFMA kernels (bf16 or fp16, D 32, 64 or 128) or SA2_ERR_UNSUPPORTED; also takes
-                                       their pre-pass kernels whenever the window sizes allow, whatever the
+#define SA2_FLAG_FORCE_MFMA 2u      /* MFMA kernels (bf16 or fp16 with D 32, 64, 128 or 256; fp32 with D 32, 64 or 128;
+                                       16-byte aligned rows) or SA2_ERR_UNSUPPORTED; also takes the pre-pass kernels
+                                       of the 16-bit D 32/64/128 path whenever the window sizes allow, whatever the
                                        problem size (SA2_FLAG_AUTO leaves them out for small grids) */
 
 /* Tensor order of the `strides` argument (3 int64 per tensor: batch, sequence, head). */
@@ -65,11 +66,11 @@ int sa2_version(void);
 /* Static, NUL-terminated description of a status code. */
 const char* sa2_strerror(int status);
 
-/* 1 if sa2_forward would take the MFMA kernels for this problem under SA2_FLAG_AUTO
- * (given 16-byte aligned rows), 0 if it would take the generic kernels.  It answers for
- * the forward only: sa2_backward additionally falls back to the generic kernels for
- * D = 32 problems whose K' window exceeds what its on-chip kernels hold (several hundred
- * positions). */
+/* 1 if sa2_forward would take MFMA kernels for this problem under SA2_FLAG_AUTO
+ * (given 16-byte aligned rows), 0 if it would take the fp32-FMA kernels.  It answers for
+ * the forward only: sa2_backward additionally falls back to the fp32-FMA kernels when the K' window
+ * exceeds what its on-chip accumulators hold (16-bit D = 32: w2 > 739; D = 256: w2 > 82; fp32:
+ * w2 > 86, 378, 913 at D = 128, 64, 32). */
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype);
 
 /*
