@@ -14,7 +14,9 @@
 // kernel adds up (a query gets partials from at most 2 + w2/32 workgroups, summed in a
 // fixed order: bitwise reproducible).
 //
-// Eight wavefronts, two per SIMD, form four pairs that each hold one unit per round and
+// Eight wavefronts, two per SIMD, form four pairs that each hold one unit per round (two
+// consecutive deltas at head_dim 32 and 64, where the registers allow it: every K and V operand
+// read, tile request and step barrier then serves twice the MFMAs) and
 // sweep the K1/V1 window in 32-key tiles staged through a three-deep LDS ring:
 //   the "P" wavefront computes S^T = K1.Q~^T, P = exp2(S - LSE), hands P (16 bit) to its
 //       partner through LDS and accumulates R^T += V1^T.P^T;
@@ -38,7 +40,8 @@ __device__ __forceinline__ int kp_recompute_here(int x) {
     return x;
 }
 
-template <int D>
+// U: units (consecutive deltas) a wavefront pair holds per round
+template <int D, int U = 1>
 struct KpCfg {
     static constexpr int DK = D / 16;
     static constexpr int DT = D / 32;
@@ -55,7 +58,7 @@ struct KpCfg {
     static constexpr int NSTAGE = 3;
     static constexpr int RS = D + 8;           // raw row / slab row stride (bf16)
     static constexpr int AS = D + 4;           // fp32 accumulator row stride
-    static constexpr int PX_BYTES = NPAIR * 2 * 64 * 32;         // P hand-over, double buffered
+    static constexpr int PX_BYTES = NPAIR * 2 * U * 64 * 32;     // P hand-over, double buffered
     static constexpr size_t LDS_LIMIT = 160 * 1024;
     // raw = true: the q and dO rows the workgroup touches are copied to LDS; otherwise the
     // wavefronts read them from global memory once per unit
@@ -81,14 +84,19 @@ struct KpCfg {
 // results go where the main kernel (launched next with left = 1) picks them up: dK'
 // and dV' in the element type in the output tensors, the dQ contribution as fp32 in rows
 // w2 .. w2+31 of the block's dQ partial.  The main kernel then handles delta < w2.
-template <class E, int D, bool RAW, bool LEFT>
+//
+// U = 2 (head_dim 32 and 64, where the registers allow it): a pair holds two consecutive deltas per round, so
+// that every K and V operand read, every tile request and every step barrier serves twice the MFMAs.
+template <class E, int D, bool RAW, bool LEFT, int U>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int left) {
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
     constexpr bool raw = RAW;
     static_assert(!(RAW && LEFT), "the pre-pass keeps no row copies in LDS");
-    using C = KpCfg<D>;
+    static_assert(!LEFT || U == 1, "the pre-pass holds one unit per pair");
+    using C = KpCfg<D, U>;
+    constexpr int UPR = NPAIR * U;                            // units per round
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int RQ = BQ + w2;                                   // query rows this workgroup touches
@@ -134,17 +142,17 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     // the unit delta = w2 exists for this block and the pre-pass took it
     const bool has_left = left && !LEFT && k0 + w2 <= N - 1;
     const int n_units = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1 - (has_left ? 1 : 0);
-    const int nrounds = LEFT ? 1 : (n_units + NPAIR - 1) / NPAIR;
+    const int nrounds = LEFT ? 1 : (n_units + UPR - 1) / UPR;
     // Tiles a round sweeps: from the first tile of its smallest delta to the last tile of its
     // largest one (tile indices relative to jt_lo).
     auto round_first = [&](int round) {
         if (LEFT) return 0;
-        const int i_min = k0 + round * NPAIR;
+        const int i_min = k0 + round * UPR;
         return (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo;
     };
     auto round_last = [&](int round) {
         if (LEFT) return nt - 1;
-        const int dl = (round + 1) * NPAIR - 1 < n_units - 1 ? (round + 1) * NPAIR - 1 : n_units - 1;
+        const int dl = (round + 1) * UPR - 1 < n_units - 1 ? (round + 1) * UPR - 1 : n_units - 1;
         const int i_max = k0 + dl + BQ - 1 < N - 1 ? k0 + dl + BQ - 1 : N - 1;
         return i_max / TJ - jt_lo;
     };
@@ -238,7 +246,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     };
     const float qscale = p.scale * LOG2E;
     const uint32_t smem_addr = lds_address(smem);
-    const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * 64 * 32 + lane * 32);
+    const uint32_t px_addr = lds_address(px) + (uint32_t)(pr * 2 * U * 64 * 32 + lane * 32);
     const uint32_t row_lane = (uint32_t)((ln / C::RPW) * C::GROUP + (hf * C::RPW + ln % C::RPW) * 16);   // row operand
     const uint32_t col_lane = lds_group_column_lane_offset<C::RPW, C::GROUP>(lane);                      // transposed operand
     constexpr uint32_t KKB = 32 * C::RPW, DTB = 64 * C::RPW;      // operand strides of a k-step / a 32-column block
@@ -293,103 +301,128 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     if (role == 0) {
         // =============================== P wavefronts ================================
         for (int round = 0; round < nrounds; ++round) {
-            const int delta = LEFT ? w2 : round * NPAIR + pr;
-            const bool ok = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta < n_units;
-            const int i = k0 + ln + delta;
-            const bool row_ok = i < N;
-            const int i_min = k0 + delta;
-            const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
-            const bool rows_full = i_min + BQ - 1 < N;
-            const int sa = ok ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;     // first and last tile of the unit
-            const int sb = ok ? i_max / TJ - jt_lo : -1;
-            floatx16 racc[C::DT];
+            int delta[U], i_min[U], i_max[U], sa[U], sb[U];
+            bool ok[U], row_ok[U], rows_full[U];
+            floatx16 racc[U][C::DT];
+            X8 qf[U][C::DK];
+            floatx16 negl[U];
+            const int i_of_lane = k0 + ln;
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt)
+            for (int u = 0; u < U; ++u) {
+                delta[u] = LEFT ? w2 : round * UPR + pr * U + u;
+                ok[u] = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta[u] < n_units;
+                row_ok[u] = i_of_lane + delta[u] < N;
+                i_min[u] = k0 + delta[u];
+                i_max[u] = (i_min[u] + BQ - 1 < N ? i_min[u] + BQ - 1 : N - 1);
+                rows_full[u] = i_min[u] + BQ - 1 < N;
+                sa[u] = ok[u] ? (i_min[u] - w1 > 0 ? i_min[u] - w1 : 0) / TJ - jt_lo : nt;     // first and last tile of the unit
+                sb[u] = ok[u] ? i_max[u] / TJ - jt_lo : -1;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) racc[dt][v] = 0.f;
-            X8 qf[C::DK];
-            float lse2 = 0.f;
-            {
-                const uint16_t* qrow = q_row(ln + delta) + hf * 8;
-                const uint16_t* krow = k2_row() + hf * 8;
-                uint4 qav[C::DK], kxv[C::DK];       // all reads of the two rows first
+                for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) qav[kk] = *(const uint4*)(qrow + kk * 16);
+                    for (int v = 0; v < 16; ++v) racc[u][dt][v] = 0.f;
+                float lse2 = 0.f;
+                {
+                    const uint16_t* qrow = q_row(ln + delta[u]) + hf * 8;
+                    const uint16_t* krow = k2_row() + hf * 8;
+                    uint4 qav[C::DK], kxv[C::DK];       // all reads of the two rows first
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) kxv[kk] = *(const uint4*)(krow + kk * 16);
+                    for (int kk = 0; kk < C::DK; ++kk) qav[kk] = *(const uint4*)(qrow + kk * 16);
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) {
-                    const uint4 qa = qav[kk];
-                    const uint4 kx = kxv[kk];
-                    const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
-                    const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w};
-                    X8 r;
+                    for (int kk = 0; kk < C::DK; ++kk) kxv[kk] = *(const uint4*)(krow + kk * 16);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        r[2 * t] = (EL)(E::lo(qw[t]) * (E::lo(kw[t]) + p.k2_bias) * qscale);
-                        r[2 * t + 1] = (EL)(E::hi(qw[t]) * (E::hi(kw[t]) + p.k2_bias) * qscale);
+                    for (int kk = 0; kk < C::DK; ++kk) {
+                        const uint4 qa = qav[kk];
+                        const uint4 kx = kxv[kk];
+                        const uint32_t qw[4] = {qa.x, qa.y, qa.z, qa.w};
+                        const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w};
+                        X8 r;
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            r[2 * t] = (EL)(E::lo(qw[t]) * (E::lo(kw[t]) + p.k2_bias) * qscale);
+                            r[2 * t + 1] = (EL)(E::hi(qw[t]) * (E::hi(kw[t]) + p.k2_bias) * qscale);
+                        }
+                        qf[u][kk] = r;
                     }
-                    qf[kk] = r;
+                    const int iu = i_of_lane + delta[u];
+                    if constexpr (LEFT) lse2 = p.lse[(int64_t)bh * N + (iu < N ? iu : N - 1)] * LOG2E;
+                    else if (ok[u]) lse2 = lse_s[ln + delta[u]];
                 }
-                if constexpr (LEFT) lse2 = p.lse[(int64_t)bh * N + (i < N ? i : N - 1)] * LOG2E;
-                else if (ok) lse2 = lse_s[ln + delta];
-            }
-            floatx16 negl;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) negl[v] = -lse2;
+                for (int v = 0; v < 16; ++v) negl[u][v] = -lse2;
+            }
             const int s_end = round_last(round);
             for (int s = round_first(round); s <= s_end; ++s) {
                 begin_step();
-                if (s >= sa && s <= sb) {
+                bool in[U];
+                bool any = false;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    in[u] = s >= sa[u] && s <= sb[u];
+                    any |= in[u];
+                }
+                if (any) {
                     const int j0 = (jt_lo + s) * TJ;
                     const uint32_t ks_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u;
                     X8 ka[C::DK];
 #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) ka[kk] = lds_read_x8<X8>(ks_addr + row_lane + kk * KKB);
-                    floatx16 sh;
-                    const bool plain = rows_full && j0 + TJ - 1 <= i_min && j0 >= i_max - w1;
-                    if (__builtin_expect(plain, 1)) {
-                        sh = E::mfma(ka[0], qf[0], negl, 0, 0, 0);
-                    } else {
-                        asm volatile("" ::: "memory");
-                        // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
-                        const int hi = i - j0 - 4 * hf, lo = hi - w1;
-                        floatx16 ct;
+                    X8 pb[U][2];
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int c = 8 * (v >> 2) + (v & 3);
-                            ct[v] = (row_ok & (c <= hi) & (c >= lo)) ? negl[0] : -INFINITY;
+                    for (int u = 0; u < U; ++u) {
+                        if (!in[u]) continue;
+                        floatx16 sh;
+                        const bool plain = rows_full[u] && j0 + TJ - 1 <= i_min[u] && j0 >= i_max[u] - w1;
+                        if (__builtin_expect(plain, 1)) {
+                            sh = E::mfma(ka[0], qf[u][0], negl[u], 0, 0, 0);
+                        } else {
+                            asm volatile("" ::: "memory");
+                            // element v of this lane is key j0 + 8*(v/4) + 4*hf + v%4
+                            const int hi = i_of_lane + delta[u] - j0 - 4 * hf, lo = hi - w1;
+                            floatx16 ct;
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                const int c = 8 * (v >> 2) + (v & 3);
+                                ct[v] = (row_ok[u] & (c <= hi) & (c >= lo)) ? negl[u][0] : -INFINITY;
+                            }
+                            sh = E::mfma(ka[0], qf[u][0], ct, 0, 0, 0);
                         }
-                        sh = E::mfma(ka[0], qf[0], ct, 0, 0, 0);
+#pragma unroll
+                        for (int kk = 1; kk < C::DK; ++kk)
+                            sh = E::mfma(ka[kk], qf[u][kk], sh, 0, 0, 0);
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                            for (int t = 0; t < 8; ++t) pb[u][ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
                     }
-#pragma unroll
-                    for (int kk = 1; kk < C::DK; ++kk)
-                        sh = E::mfma(ka[kk], qf[kk], sh, 0, 0, 0);
-                    X8 pb[2];
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                        for (int t = 0; t < 8; ++t) pb[ks][t] = (EL)fast_exp2(sh[ks * 8 + t]);
                     lds_half_operand vh[4 * C::DT];
                     issue_tr(ks_addr + (uint32_t)C::TILE_BYTES + col_lane, vh);
-                    {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        if (!in[u]) continue;
                         // opaque stores: the compiler would wait for the tile request in flight
-                        const uint32_t a = px_addr + (uint32_t)((g & 1) * 64 * 32);
-                        asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16" ::"v"(a), "v"(pb[0]), "v"(pb[1]) : "memory");
+                        const uint32_t a = px_addr + (uint32_t)(((g & 1) * U + u) * 64 * 32);
+                        asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16" ::"v"(a), "v"(pb[u][0]), "v"(pb[u][1]) : "memory");
                     }
                     lds_settle(vh);
 #pragma unroll
-                    for (int dt = 0; dt < C::DT; ++dt)
+                    for (int u = 0; u < U; ++u) {
+                        if (!in[u]) continue;
 #pragma unroll
-                        for (int ks = 0; ks < 2; ++ks)
-                            racc[dt] = E::mfma(lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]),
-                                                                               pb[ks], racc[dt], 0, 0, 0);
+                        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                            for (int ks = 0; ks < 2; ++ks)
+                                racc[u][dt] = E::mfma(lds_join<X8>(vh[4 * dt + 2 * ks], vh[4 * dt + 2 * ks + 1]),
+                                                      pb[u][ks], racc[u][dt], 0, 0, 0);
+                    }
                 }
                 advance();
             }
             // dV'[k] += R[(k+delta, k)] * dO[k+delta]
-            if (ok) {
-                const uint16_t* drow = do_row(ln + delta) + 4 * hf;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (!ok[u]) continue;
+                const uint16_t* drow = do_row(ln + delta[u]) + 4 * hf;
                 uint2 dx[4 * C::DT];               // the dO row, read in one batch
 #pragma unroll
                 for (int e = 0; e < 4 * C::DT; ++e) dx[e] = *(const uint2*)(drow + (e >> 2) * 32 + 8 * (e & 3));
@@ -398,15 +431,15 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
                         const uint2 x = dx[4 * dt + g4];
-                        pacc[dt][4 * g4 + 0] += racc[dt][4 * g4 + 0] * E::lo(x.x);
-                        pacc[dt][4 * g4 + 1] += racc[dt][4 * g4 + 1] * E::hi(x.x);
-                        pacc[dt][4 * g4 + 2] += racc[dt][4 * g4 + 2] * E::lo(x.y);
-                        pacc[dt][4 * g4 + 3] += racc[dt][4 * g4 + 3] * E::hi(x.y);
+                        pacc[dt][4 * g4 + 0] += racc[u][dt][4 * g4 + 0] * E::lo(x.x);
+                        pacc[dt][4 * g4 + 1] += racc[u][dt][4 * g4 + 1] * E::hi(x.x);
+                        pacc[dt][4 * g4 + 2] += racc[u][dt][4 * g4 + 2] * E::lo(x.y);
+                        pacc[dt][4 * g4 + 3] += racc[u][dt][4 * g4 + 3] * E::hi(x.y);
                     }
             }
             if constexpr (LEFT) {
                 // pre-pass: dV' of the unit goes to the output tensor as it is
-                if (ok && p.dv2.p && k0 + ln < N) {
+                if (ok[0] && p.dv2.p && k0 + ln < N) {
                     uint16_t* dst = (uint16_t*)p.dv2.p + p.dv2.off(b, k0 + ln, h) + 4 * hf;
 #pragma unroll
                     for (int dt = 0; dt < C::DT; ++dt)
@@ -430,91 +463,119 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     } else {
         // =============================== dS wavefronts ===============================
         for (int round = 0; round < nrounds; ++round) {
-            const int delta = LEFT ? w2 : round * NPAIR + pr;
-            const bool ok = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta < n_units;
-            const int i_min = k0 + delta;
-            const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
-            const int sa = ok ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;
-            const int sb = ok ? i_max / TJ - jt_lo : -1;
-            floatx16 gacc[C::DT];
+            int delta[U], sa[U], sb[U];
+            bool ok[U];
+            floatx16 gacc[U][C::DT];
+            X8 dof[U][C::DK];
+            floatx16 dp_prev[U], negd[U];
 #pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt)
+            for (int u = 0; u < U; ++u) {
+                delta[u] = LEFT ? w2 : round * UPR + pr * U + u;
+                ok[u] = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta[u] < n_units;
+                const int i_min = k0 + delta[u];
+                const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
+                sa[u] = ok[u] ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;
+                sb[u] = ok[u] ? i_max / TJ - jt_lo : -1;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) gacc[dt][v] = 0.f;
-            X8 dof[C::DK];
-            float dsum = 0.f;
-            {
-                const uint16_t* drow = do_row(ln + delta) + hf * 8;
-                const uint16_t* vrow = v2_row() + hf * 8;
-                uint4 dav[C::DK], vxv[C::DK];       // all reads of the two rows first
+                for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) dav[kk] = *(const uint4*)(drow + kk * 16);
+                    for (int v = 0; v < 16; ++v) gacc[u][dt][v] = 0.f;
+                float dsum = 0.f;
+                {
+                    const uint16_t* drow = do_row(ln + delta[u]) + hf * 8;
+                    const uint16_t* vrow = v2_row() + hf * 8;
+                    uint4 dav[C::DK], vxv[C::DK];       // all reads of the two rows first
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) vxv[kk] = *(const uint4*)(vrow + kk * 16);
+                    for (int kk = 0; kk < C::DK; ++kk) dav[kk] = *(const uint4*)(drow + kk * 16);
 #pragma unroll
-                for (int kk = 0; kk < C::DK; ++kk) {
-                    const uint4 da = dav[kk];
-                    const uint4 vx = vxv[kk];
-                    const uint32_t dw[4] = {da.x, da.y, da.z, da.w};
-                    const uint32_t vw[4] = {vx.x, vx.y, vx.z, vx.w};
-                    X8 r;
+                    for (int kk = 0; kk < C::DK; ++kk) vxv[kk] = *(const uint4*)(vrow + kk * 16);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        r[2 * t] = (EL)(E::lo(dw[t]) * (E::lo(vw[t]) + p.v2_bias));
-                        r[2 * t + 1] = (EL)(E::hi(dw[t]) * (E::hi(vw[t]) + p.v2_bias));
+                    for (int kk = 0; kk < C::DK; ++kk) {
+                        const uint4 da = dav[kk];
+                        const uint4 vx = vxv[kk];
+                        const uint32_t dw[4] = {da.x, da.y, da.z, da.w};
+                        const uint32_t vw[4] = {vx.x, vx.y, vx.z, vx.w};
+                        X8 r;
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            r[2 * t] = (EL)(E::lo(dw[t]) * (E::lo(vw[t]) + p.v2_bias));
+                            r[2 * t + 1] = (EL)(E::hi(dw[t]) * (E::hi(vw[t]) + p.v2_bias));
+                        }
+                        dof[u][kk] = r;
                     }
-                    dof[kk] = r;
+                    if constexpr (LEFT) dsum = p.dsum[(int64_t)bh * N + (i_min + ln < N ? i_min + ln : N - 1)];
+                    else if (ok[u]) dsum = dsum_s[ln + delta[u]];
                 }
-                if constexpr (LEFT) dsum = p.dsum[(int64_t)bh * N + (i_min + ln < N ? i_min + ln : N - 1)];
-                else if (ok) dsum = dsum_s[ln + delta];
-            }
-            floatx16 dp_prev, negd;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) { dp_prev[v] = 0.f; negd[v] = -dsum; }
-            // dS of the tile handled in the previous step and its G MFMAs
-            auto consume = [&]() {
+                for (int v = 0; v < 16; ++v) { dp_prev[u][v] = 0.f; negd[u][v] = -dsum; }
+            }
+            // dS of the tile handled in the previous step (tile index sp) and its G MFMAs
+            auto consume = [&](int sp) {
                 typedef const X8 __attribute__((address_space(3)))* lds_b8;
-                const uint32_t a = px_addr + (uint32_t)(((g - 1) & 1) * 64 * 32);
-                const X8 p0 = *(lds_b8)(uintptr_t)a, p1 = *(lds_b8)(uintptr_t)(a + 16);
+                X8 p0[U], p1[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t a = px_addr + (uint32_t)((((g - 1) & 1) * U + u) * 64 * 32);
+                    p0[u] = *(lds_b8)(uintptr_t)a;
+                    p1[u] = *(lds_b8)(uintptr_t)(a + 16);
+                }
                 const int pb = buf == 0 ? C::NSTAGE - 1 : buf - 1;
                 lds_half_operand kh[4 * C::DT];
                 issue_tr(smem_addr + (uint32_t)(pb * C::STAGE) * 2u + col_lane, kh);
                 lds_settle(kh);
-                X8 dsb[2];
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    dsb[0][t] = (EL)((float)p0[t] * dp_prev[t]);
-                    dsb[1][t] = (EL)((float)p1[t] * dp_prev[8 + t]);
+                for (int u = 0; u < U; ++u) {
+                    if (U > 1 && !(sp >= sa[u] && sp <= sb[u])) continue;
+                    X8 dsb[2];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        dsb[0][t] = (EL)((float)p0[u][t] * dp_prev[u][t]);
+                        dsb[1][t] = (EL)((float)p1[u][t] * dp_prev[u][8 + t]);
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks)
+                            gacc[u][dt] = E::mfma(lds_join<X8>(kh[4 * dt + 2 * ks], kh[4 * dt + 2 * ks + 1]),
+                                                  dsb[ks], gacc[u][dt], 0, 0, 0);
                 }
+            };
+            auto any_in = [&](int sx) {
+                bool r = false;
 #pragma unroll
-                for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
-                        gacc[dt] = E::mfma(lds_join<X8>(kh[4 * dt + 2 * ks], kh[4 * dt + 2 * ks + 1]),
-                                                                           dsb[ks], gacc[dt], 0, 0, 0);
+                for (int u = 0; u < U; ++u) r |= sx >= sa[u] && sx <= sb[u];
+                return r;
             };
             const int s_end = round_last(round);
             for (int s = round_first(round); s <= s_end; ++s) {
                 begin_step();
-                if (s - 1 >= sa && s - 1 <= sb) consume();
-                if (s >= sa && s <= sb) {
+                if (any_in(s - 1)) consume(s - 1);
+                if (any_in(s)) {
                     const uint32_t vs_addr = smem_addr + (uint32_t)(buf * C::STAGE) * 2u + (uint32_t)C::TILE_BYTES;
                     X8 va[C::DK];
 #pragma unroll
                     for (int kk = 0; kk < C::DK; ++kk) va[kk] = lds_read_x8<X8>(vs_addr + row_lane + kk * KKB);
-                    dp_prev = E::mfma(va[0], dof[0], negd, 0, 0, 0);
 #pragma unroll
-                    for (int kk = 1; kk < C::DK; ++kk)
-                        dp_prev = E::mfma(va[kk], dof[kk], dp_prev, 0, 0, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
+                    for (int u = 0; u < U; ++u) {
+                        if (!(s >= sa[u] && s <= sb[u])) continue;
+                        dp_prev[u] = E::mfma(va[0], dof[u][0], negd[u], 0, 0, 0);
+#pragma unroll
+                        for (int kk = 1; kk < C::DK; ++kk)
+                            dp_prev[u] = E::mfma(va[kk], dof[u][kk], dp_prev[u], 0, 0, 0);
+                    }
+                    if constexpr (U == 1) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, C::DK, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, C::DK, 0);
+                    }
                 }
                 advance();
             }
-            if (s_end >= sa && s_end <= sb) consume();
+            if (any_in(s_end)) consume(s_end);
             // dK'[k] += G[(k+delta, k)] * q[k+delta]   (scale applied at the end)
-            if (ok) {
-                const uint16_t* qrow = q_row(ln + delta) + 4 * hf;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (!ok[u]) continue;
+                const uint16_t* qrow = q_row(ln + delta[u]) + 4 * hf;
                 uint2 qx[4 * C::DT];               // the q row, read in one batch
 #pragma unroll
                 for (int e = 0; e < 4 * C::DT; ++e) qx[e] = *(const uint2*)(qrow + (e >> 2) * 32 + 8 * (e & 3));
@@ -523,16 +584,16 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
                         const uint2 x = qx[4 * dt + g4];
-                        pacc[dt][4 * g4 + 0] += gacc[dt][4 * g4 + 0] * E::lo(x.x);
-                        pacc[dt][4 * g4 + 1] += gacc[dt][4 * g4 + 1] * E::hi(x.x);
-                        pacc[dt][4 * g4 + 2] += gacc[dt][4 * g4 + 2] * E::lo(x.y);
-                        pacc[dt][4 * g4 + 3] += gacc[dt][4 * g4 + 3] * E::hi(x.y);
+                        pacc[dt][4 * g4 + 0] += gacc[u][dt][4 * g4 + 0] * E::lo(x.x);
+                        pacc[dt][4 * g4 + 1] += gacc[u][dt][4 * g4 + 1] * E::hi(x.x);
+                        pacc[dt][4 * g4 + 2] += gacc[u][dt][4 * g4 + 2] * E::lo(x.y);
+                        pacc[dt][4 * g4 + 3] += gacc[u][dt][4 * g4 + 3] * E::hi(x.y);
                     }
             }
             if constexpr (LEFT) {
                 // pre-pass: dK' of the unit goes to the output tensor, its dQ
                 // contribution G * k2~ (unscaled) to rows w2 .. w2+31 of the block's dQ partial
-                if (ok && k0 + ln < N) {
+                if (ok[0] && k0 + ln < N) {
                     if (p.dk2.p) {
                         uint16_t* dst = (uint16_t*)p.dk2.p + p.dk2.off(b, k0 + ln, h) + 4 * hf;
 #pragma unroll
@@ -546,7 +607,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                             }
                     }
                 }
-                if (ok && want_dq) {
+                if (ok[0] && want_dq) {
                     // (rows of keys past the end of the sequence carry zeros: their G is zero)
                     float* dst = dq_part + (((int64_t)bh * nkb_all + kb) * RQ + w2 + ln) * D + 4 * hf;
                     const uint16_t* krow = k2_row() + 4 * hf;
@@ -559,32 +620,34 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                         for (int g4 = 0; g4 < 4; ++g4) {
                             const uint2 x = kx[4 * dt + g4];
                             float4 a;
-                            a.x = gacc[dt][4 * g4 + 0] * (E::lo(x.x) + p.k2_bias);
-                            a.y = gacc[dt][4 * g4 + 1] * (E::hi(x.x) + p.k2_bias);
-                            a.z = gacc[dt][4 * g4 + 2] * (E::lo(x.y) + p.k2_bias);
-                            a.w = gacc[dt][4 * g4 + 3] * (E::hi(x.y) + p.k2_bias);
+                            a.x = gacc[0][dt][4 * g4 + 0] * (E::lo(x.x) + p.k2_bias);
+                            a.y = gacc[0][dt][4 * g4 + 1] * (E::hi(x.x) + p.k2_bias);
+                            a.z = gacc[0][dt][4 * g4 + 2] * (E::lo(x.y) + p.k2_bias);
+                            a.w = gacc[0][dt][4 * g4 + 3] * (E::hi(x.y) + p.k2_bias);
                             *(float4*)(dst + dt * 32 + 8 * g4) = a;
                         }
                 }
                 return;
             }
             if (want_dq) {
-                // dQ contribution of the unit: dqacc[ln + delta][:] += G * k2~.  The four dS
+                // dQ contribution of the units: dqacc[ln + delta][:] += G * k2~.  The four dS
                 // wavefronts add into the shared fp32 accumulator (scale is applied when the
                 // partial is written out) in four phases; in phase t
                 // wavefront pr owns the 16-column blocks (pr + t) % 4 (and that + 4 when D = 128),
                 // so no two wavefronts touch an element at the same time and every element
-                // receives its contributions in a fixed order.
+                // receives its contributions in a fixed order (a wavefront's units one after the other).
                 auto add_dq = [&](auto PR, auto BIASED) {
                     constexpr int P0 = decltype(PR)::value;
                     constexpr bool WITH_BIAS = decltype(BIASED)::value;
                     const int tid_q = kp_recompute_here(threadIdx.x);
                     const int ln_q = tid_q & 31, hf_q = (tid_q >> 5) & 1;
-                    float* arow = dqacc + (ln_q + delta) * C::AS + 4 * hf_q;
                     const uint16_t* krow = k2_s + ln_q * C::RS + 4 * hf_q;      // (main kernel only)
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        if (ok) {
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            if (!ok[u]) continue;
+                            float* arow = dqacc + (ln_q + delta[u]) * C::AS + 4 * hf_q;
                             constexpr int NV = C::DK / 2;             // float4 slots of this phase
                             float4 a[NV];
                             uint2 x[NV];
@@ -605,12 +668,16 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                             for (int e = 0; e < NV; ++e) {
                                 const int dt = slot_dt(e), g4 = slot_g4(e);
                                 const float kb = WITH_BIAS ? p.k2_bias : 0.f;
-                                a[e].x += gacc[dt][4 * g4 + 0] * (E::lo(x[e].x) + kb);
-                                a[e].y += gacc[dt][4 * g4 + 1] * (E::hi(x[e].x) + kb);
-                                a[e].z += gacc[dt][4 * g4 + 2] * (E::lo(x[e].y) + kb);
-                                a[e].w += gacc[dt][4 * g4 + 3] * (E::hi(x[e].y) + kb);
+                                a[e].x += gacc[u][dt][4 * g4 + 0] * (E::lo(x[e].x) + kb);
+                                a[e].y += gacc[u][dt][4 * g4 + 1] * (E::hi(x[e].x) + kb);
+                                a[e].z += gacc[u][dt][4 * g4 + 2] * (E::lo(x[e].y) + kb);
+                                a[e].w += gacc[u][dt][4 * g4 + 3] * (E::hi(x[e].y) + kb);
                                 *(float4*)(arow + dt * 32 + 8 * g4) = a[e];
                             }
+                            // (the second unit's rows overlap the first one's, shifted by one: its reads
+                            // must see the first unit's writes, which the same lanes' program order does not
+                            // give across lanes)
+                            if constexpr (U > 1) __builtin_amdgcn_wave_barrier();
                         }
                         if (t < 3) __syncthreads();
                     }
@@ -745,9 +812,14 @@ __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const f
     *(uint4*)((uint16_t*)p.dq.p + p.dq.off(b, i, h) + c0) = o.u;
 }
 
+// units per pair and round of the main kernel
+template <int D>
+constexpr int kp_units() { return D <= 64 ? 2 : 1; }
+
 template <class E, int D>
 int launch_kp(const Problem& p, hipStream_t st) {
-    using C = KpCfg<D>;
+    constexpr int U = kp_units<D>();
+    using C = KpCfg<D, U>;
     const int nkb = (p.N + BQ - 1) / BQ;
     const int64_t total = (int64_t)nkb * p.B * p.H;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
@@ -759,18 +831,18 @@ int launch_kp(const Problem& p, hipStream_t st) {
     // (unless the grid is so small that a further launch costs more than the lone round)
     const int left = (p.w2 >= NPAIR && p.w2 % NPAIR == 0 && (p.force_prepass || total >= 768)) ? 1 : 0;
     if (left) {
-        const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + C::PX_BYTES;
+        const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + KpCfg<D, 1>::PX_BYTES;
         const int ngrp = (nkb + NPAIR - 1) / NPAIR;
         const int64_t total_left = (int64_t)ngrp * p.B * p.H;
-        if (!allow_full_lds((const void*)mfma_bwd_kp_kernel<E, D, false, true>)) return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, true>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
+        if (!allow_full_lds((const void*)mfma_bwd_kp_kernel<E, D, false, true, 1>)) return SA2_ERR_LAUNCH_FAILED;
+        hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, true, 1>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
                            (int)total_left, part, 0);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
-    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<E, D, true, false> : (const void*)mfma_bwd_kp_kernel<E, D, false, false>;
+    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<E, D, true, false, U> : (const void*)mfma_bwd_kp_kernel<E, D, false, false, U>;
     if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
-    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, true, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
-    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
+    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, true, false, U>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
+    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false, U>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (p.dq.p) {
         const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
@@ -784,7 +856,8 @@ int launch_kp(const Problem& p, hipStream_t st) {
 }  // namespace
 
 bool kp_fits(int D, int w2) {
-    return D == 128 ? KpCfg<128>::fits(w2) : D == 64 ? KpCfg<64>::fits(w2) : D == 32 ? KpCfg<32>::fits(w2) : false;
+    return D == 128 ? KpCfg<128, kp_units<128>()>::fits(w2) : D == 64 ? KpCfg<64, kp_units<64>()>::fits(w2)
+           : D == 32 ? KpCfg<32, kp_units<32>()>::fits(w2) : false;
 }
 
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {
