@@ -812,13 +812,13 @@ __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const f
     *(uint4*)((uint16_t*)p.dq.p + p.dq.off(b, i, h) + c0) = o.u;
 }
 
-// units per pair and round of the main kernel
+// units per pair and round of the main kernel: two at head_dim 32 and 64 while the doubled P hand-over
+// still leaves room for the dQ accumulator, else one
 template <int D>
 constexpr int kp_units() { return D <= 64 ? 2 : 1; }
 
-template <class E, int D>
-int launch_kp(const Problem& p, hipStream_t st) {
-    constexpr int U = kp_units<D>();
+template <class E, int D, int U>
+int launch_kp_units(const Problem& p, hipStream_t st) {
     using C = KpCfg<D, U>;
     const int nkb = (p.N + BQ - 1) / BQ;
     const int64_t total = (int64_t)nkb * p.B * p.H;
@@ -853,11 +853,18 @@ int launch_kp(const Problem& p, hipStream_t st) {
     return SA2_OK;
 }
 
+template <class E, int D>
+int launch_kp(const Problem& p, hipStream_t st) {
+    if constexpr (kp_units<D>() == 2) {
+        if (KpCfg<D, 2>::fits(p.w2)) return launch_kp_units<E, D, 2>(p, st);
+    }
+    return launch_kp_units<E, D, 1>(p, st);
+}
+
 }  // namespace
 
 bool kp_fits(int D, int w2) {
-    return D == 128 ? KpCfg<128, kp_units<128>()>::fits(w2) : D == 64 ? KpCfg<64, kp_units<64>()>::fits(w2)
-           : D == 32 ? KpCfg<32, kp_units<32>()>::fits(w2) : false;
+    return D == 128 ? KpCfg<128, 1>::fits(w2) : D == 64 ? KpCfg<64, 1>::fits(w2) : D == 32 ? KpCfg<32, 1>::fits(w2) : false;
 }
 
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {

@@ -34,6 +34,10 @@ SMALL = [  # B, N, H, D, w1, w2, k2_bias, v2_bias
     (1, 150, 1, 128, 20, 65, 0.0, 0.0),      # first K' window beyond the K-side on-chip kernel (64 is its last)
     (1, 190, 1, 128, 12, 113, 0.0, 0.0),     # last K' window of the K'-side on-chip kernel
     (1, 190, 1, 128, 12, 114, 0.0, 0.0),     # first one beyond it
+    (1, 350, 1, 64, 12, 304, 0.0, 0.0),      # head_dim 64: last K' window with two deltas per wavefront pair
+    (1, 350, 1, 64, 12, 305, 0.1, 0.0),      # first with one delta per pair
+    (1, 390, 1, 64, 9, 362, 0.0, 0.0),       # last K' window of the K'-side on-chip kernel at head_dim 64
+    (1, 390, 1, 64, 9, 363, 0.0, 0.0),       # first one beyond it
 ]
 
 
