@@ -98,14 +98,13 @@ bool wide_bwd_supported(int D, int w2, int dtype);
 size_t wide_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 int launch_wide_fwd(const Problem& p, int dtype, hipStream_t st);
 int launch_wide_bwd(const Problem& p, int dtype, hipStream_t st);
-// K'-side backward kernel (dQ, dK', dV') that keeps its partial sums on chip
-bool kp_fits(int D, int w2);
+// K'-side backward kernel (dQ, dK', dV') that keeps its partial sums on chip (K' windows too wide for
+// that are cut into segments of deltas, one workgroup each)
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2);
 int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st);
 // K-side backward kernel (dK, dV) with paired wavefronts; for small grids it splits a key block's
 // query blocks over several workgroups, whose fp32 partial sums lie in the workspace behind the
-// K'-side part (kp_side_scratch_bytes)
-bool kv_fits(int D, int w2);
+// K'-side part (kp_side_scratch_bytes); K' windows too wide for its LDS rows are walked in segments
 size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1);
 size_t kp_side_scratch_bytes(int B, int N, int H, int D, int w2);
 int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st);

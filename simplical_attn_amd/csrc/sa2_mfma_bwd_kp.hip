@@ -87,22 +87,30 @@ struct KpCfg {
 //
 // U = 2 (head_dim 32 and 64, where the registers allow it): a pair holds two consecutive deltas per round, so
 // that every K and V operand read, every tile request and every step barrier serves twice the MFMAs.
-template <class E, int D, bool RAW, bool LEFT, int U>
+//
+// SEG = true: a K' window too wide for the dQ accumulator in LDS is cut into nseg runs of segw deltas, one
+// workgroup per (K' block, segment); a kernel of its own so that the common case carries none of it.  Each writes its own dQ partial (rows k0 + seg*segw ..) and, when
+// nseg > 1, fp32 partial dK' and dV' to `kpart` ([dV' | dK'][nseg][B*H][N][D]) for kp_sum_kernel.
+template <class E, int D, bool RAW, bool LEFT, int U, bool SEG = false>
 __global__ __launch_bounds__(KT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int left) {
+void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int left, int nseg_arg, int segw_arg,
+                        float* __restrict__ kpart) {
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
     constexpr bool raw = RAW;
     static_assert(!(RAW && LEFT), "the pre-pass keeps no row copies in LDS");
     static_assert(!LEFT || U == 1, "the pre-pass holds one unit per pair");
+    static_assert(!SEG || (!LEFT && !RAW), "segments: main kernel, rows from global memory");
     using C = KpCfg<D, U>;
     constexpr int UPR = NPAIR * U;                            // units per round
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
-    const int RQ = BQ + w2;                                   // query rows this workgroup touches
+    const int nseg = SEG ? nseg_arg : 1, segw = SEG ? segw_arg : w2 + 1;
+    const int w2s = segw - 1;                                 // deltas of a segment, minus one (w2 when there is one segment)
+    const int RQ = BQ + w2s;                                  // query rows this workgroup touches
     uint16_t* smem = (uint16_t*)smem_raw;                     // stage ring
     unsigned char* px = smem_raw + (size_t)C::NSTAGE * C::STAGE * 2;
-    uint16_t* q_s = (uint16_t*)(px + C::PX_BYTES);            // [RQ][RS] q rows k0 .. (when raw)
+    uint16_t* q_s = (uint16_t*)(px + C::PX_BYTES);            // [RQ][RS] q rows kq .. (when raw)
     uint16_t* do_s = q_s + RQ * C::RS;                        // [RQ][RS] dO rows      (when raw)
     uint16_t* k2_s = raw ? do_s + RQ * C::RS : q_s;           // [BQ][RS] K' rows k0 ..
     uint16_t* v2_s = k2_s + BQ * C::RS;                       // [BQ][RS] V' rows
@@ -116,15 +124,24 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const int role = wave >> 2, pr = wave & 3;                // role 0: P wavefront, 1: dS wavefront
     const int lane = tid & 63, ln = lane & 31, hf = lane >> 5;
 
-    int pid = blockIdx.x;
-    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    // Launch order: all (K' block, head) pairs of segment 0, then those of segment 1, ...: the last segment
+    // is the short one, and workgroups that alternate between long and short in launch order end up with
+    // the long ones on half of the CUs (measured: twice the time).  Within a segment consecutive blocks go
+    // to the same XCD.
+    const int per_seg = SEG ? total / nseg : total;
+    const int seg = SEG ? (int)blockIdx.x / per_seg : 0;
+    int pb = SEG ? (int)blockIdx.x - seg * per_seg : (int)blockIdx.x;
+    if ((per_seg & 7) == 0) pb = (pb & 7) * (per_seg >> 3) + (pb >> 3);
     // (in the pre-pass nkb counts groups of four K' blocks and k0 belongs to the pair)
-    const int bh = pid / nkb, kb = LEFT ? (pid - bh * nkb) * NPAIR + pr : pid - bh * nkb;
+    const int bh = pb / nkb, kb = LEFT ? (pb - bh * nkb) * NPAIR + pr : pb - bh * nkb;
     const int b = bh / p.H, h = bh - b * p.H;
     const int k0 = kb * BQ;
+    const int dlo = seg * segw;                               // first delta of the segment
+    const int dhi = dlo + w2s < w2 ? dlo + w2s : w2;          // last one
+    const int kq = k0 + dlo;                                  // query of K' row k0 at the segment's first delta
     const int k0_wg = LEFT ? (kb - pr) * BQ : k0;
     const int k0_end = LEFT ? k0_wg + NPAIR * BQ - 1 : k0 + BQ - 1;               // last K' row of the workgroup
-    const int i_hi = (int)((int64_t)k0_end + w2 < N - 1 ? k0_end + w2 : N - 1);
+    const int i_hi = (int)((int64_t)k0_end + dhi < N - 1 ? k0_end + dhi : N - 1);
     const int nkb_all = (N + BQ - 1) / BQ;
     if (LEFT && k0_wg + w2 > N - 1) return;          // none of the four blocks has the unit delta = w2
 
@@ -135,25 +152,26 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     const uint16_t* v2p = (const uint16_t*)p.v2.p + p.v2.off(b, 0, h);
     const uint16_t* dop = (const uint16_t*)p.dout.p + p.dout.off(b, 0, h);
 
-    const int i_lo = LEFT ? k0_wg + w2 : k0;                                      // first query of the workgroup
+    const int i_lo = LEFT ? k0_wg + w2 : kq;                                      // first query of the workgroup
     const int jt_lo = (i_lo - w1 > 0 ? i_lo - w1 : 0) / TJ;
     const int jt_hi = i_hi / TJ;
     const int nt = jt_hi - jt_lo + 1;
     // the unit delta = w2 exists for this block and the pre-pass took it
     const bool has_left = left && !LEFT && k0 + w2 <= N - 1;
-    const int n_units = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1 - (has_left ? 1 : 0);
+    const int nu_all = (w2 < N - 1 - k0 ? w2 : N - 1 - k0) + 1 - (has_left ? 1 : 0);      // units of the K' block
+    const int n_units = !SEG ? nu_all : nu_all - dlo < segw ? nu_all - dlo : segw;                        // of this segment (may be <= 0)
     const int nrounds = LEFT ? 1 : (n_units + UPR - 1) / UPR;
     // Tiles a round sweeps: from the first tile of its smallest delta to the last tile of its
     // largest one (tile indices relative to jt_lo).
     auto round_first = [&](int round) {
         if (LEFT) return 0;
-        const int i_min = k0 + round * UPR;
+        const int i_min = kq + round * UPR;
         return (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo;
     };
     auto round_last = [&](int round) {
         if (LEFT) return nt - 1;
         const int dl = (round + 1) * UPR - 1 < n_units - 1 ? (round + 1) * UPR - 1 : n_units - 1;
-        const int i_max = k0 + dl + BQ - 1 < N - 1 ? k0 + dl + BQ - 1 : N - 1;
+        const int i_max = kq + dl + BQ - 1 < N - 1 ? kq + dl + BQ - 1 : N - 1;
         return i_max / TJ - jt_lo;
     };
     const bool want_dq = p.dq.p != nullptr;
@@ -186,7 +204,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         constexpr int CPR = D / 8;
         for (int c = tid; c < (raw ? RQ * CPR : 0); c += KT) {
             const int row = c / CPR, col = c - row * CPR;
-            int r = k0 + row;
+            int r = kq + row;
             r = r < N ? r : N - 1;
             *(uint4*)(q_s + row * C::RS + col * 8) = *(const uint4*)(qp + (int64_t)r * p.q.sn + col * 8);
             *(uint4*)(do_s + row * C::RS + col * 8) = *(const uint4*)(dop + (int64_t)r * p.dout.sn + col * 8);
@@ -199,7 +217,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             *(uint4*)(v2_s + row * C::RS + col * 8) = *(const uint4*)(v2p + (int64_t)r * p.v2.sn + col * 8);
         }
         for (int c = tid; c < RQ; c += KT) {
-            int r = k0 + c;
+            int r = kq + c;
             r = r < N ? r : N - 1;
             lse_s[c] = p.lse[(int64_t)bh * N + r] * LOG2E;
             dsum_s[c] = p.dsum[(int64_t)bh * N + r];
@@ -217,12 +235,12 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         }
     }
 
-    // q / dO row of query k0 + rel: the LDS copy or (clamped) global memory
+    // q / dO row of query kq + rel: the LDS copy or (clamped) global memory
     auto q_row = [&](int rel) {
         if constexpr (RAW) {
             return (const uint16_t*)(q_s + rel * C::RS);
         } else {
-            const int r = k0 + rel < N ? k0 + rel : N - 1;
+            const int r = kq + rel < N ? kq + rel : N - 1;
             return qp + (int64_t)r * p.q.sn;
         }
     };
@@ -230,7 +248,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
         if constexpr (RAW) {
             return (const uint16_t*)(do_s + rel * C::RS);
         } else {
-            const int r = k0 + rel < N ? k0 + rel : N - 1;
+            const int r = kq + rel < N ? kq + rel : N - 1;
             return dop + (int64_t)r * p.dout.sn;
         }
     };
@@ -306,13 +324,13 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             floatx16 racc[U][C::DT];
             X8 qf[U][C::DK];
             floatx16 negl[U];
-            const int i_of_lane = k0 + ln;
+            const int i_of_lane = kq + ln;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 delta[u] = LEFT ? w2 : round * UPR + pr * U + u;
                 ok[u] = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta[u] < n_units;
                 row_ok[u] = i_of_lane + delta[u] < N;
-                i_min[u] = k0 + delta[u];
+                i_min[u] = kq + delta[u];
                 i_max[u] = (i_min[u] + BQ - 1 < N ? i_min[u] + BQ - 1 : N - 1);
                 rows_full[u] = i_min[u] + BQ - 1 < N;
                 sa[u] = ok[u] ? (i_min[u] - w1 > 0 ? i_min[u] - w1 : 0) / TJ - jt_lo : nt;     // first and last tile of the unit
@@ -472,7 +490,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
             for (int u = 0; u < U; ++u) {
                 delta[u] = LEFT ? w2 : round * UPR + pr * U + u;
                 ok[u] = LEFT ? (kb < nkb_all && k0 + w2 <= N - 1) : delta[u] < n_units;
-                const int i_min = k0 + delta[u];
+                const int i_min = kq + delta[u];
                 const int i_max = (i_min + BQ - 1 < N ? i_min + BQ - 1 : N - 1);
                 sa[u] = ok[u] ? (i_min - w1 > 0 ? i_min - w1 : 0) / TJ - jt_lo : nt;
                 sb[u] = ok[u] ? i_max / TJ - jt_lo : -1;
@@ -701,7 +719,7 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
     __syncthreads();
     if (want_dq) {
         constexpr int CH = D / 4;
-        float* dst = dq_part + ((int64_t)bh * nkb + kb) * RQ * D;
+        float* dst = dq_part + (((int64_t)bh * nkb + kb) * nseg + seg) * RQ * D;
         for (int it = tid_f; it < RQ * CH; it += KT) {
             const int row = it / CH, c0 = (it - row * CH) * 4;
             float4 a = *(const float4*)(dqacc + row * C::AS + c0);
@@ -768,6 +786,12 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
                 acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
             }
             const float sc = which ? p.scale : 1.f;
+            if (nseg > 1) {
+                float* dst = kpart + ((((int64_t)which * nseg + seg) * p.B * p.H + bh) * N + k) * D + c0;
+                *(float4*)dst = make_float4(acc[0] * sc, acc[1] * sc, acc[2] * sc, acc[3] * sc);
+                *(float4*)(dst + 4) = make_float4(acc[4] * sc, acc[5] * sc, acc[6] * sc, acc[7] * sc);
+                continue;
+            }
             uint16_t* dst = (uint16_t*)t.p + t.off(b, k, h) + c0;
             const uint4 x = pre[j];                                 // zeros where the pre-pass did not run
             const float part[8] = {E::lo(x.x), E::hi(x.x), E::lo(x.y), E::hi(x.y),
@@ -783,14 +807,15 @@ void mfma_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_pa
 // dQ[i] = sum of the partials of the K' blocks that reach query i, in block order.
 template <class E, int D>
 __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const float* __restrict__ dq_part, int nkb,
-                                                             int64_t items) {
+                                                             int64_t items, int nseg, int segw) {
     typedef typename E::scalar EL;
     constexpr int CH = D / 8;
     const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (it >= items) return;
     const int c0 = (int)(it % CH) * 8;
     const int64_t row = it / CH;
-    const int N = p.N, RQ = BQ + p.w2;
+    const int N = p.N, RQ = BQ + p.w2;       // queries a K' block reaches
+    const int RS = BQ + segw - 1;            // rows of one segment's partial
     const int i = (int)(row % N);
     const int bh = (int)(row / N);
     const int b = bh / p.H, h = bh - b * p.H;
@@ -800,11 +825,25 @@ __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const f
     float acc[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) acc[c] = 0.f;
+    if (nseg == 1) {
+        for (int kb = kb_lo; kb <= kb_hi; ++kb) {
+            const float* src = dq_part + (((int64_t)bh * nkb + kb) * RQ + (i - kb * BQ)) * D + c0;
+            const float4 a = *(const float4*)src, c4 = *(const float4*)(src + 4);
+            acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
+            acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
+        }
+        kb_lo = kb_hi + 1;
+    }
     for (int kb = kb_lo; kb <= kb_hi; ++kb) {
-        const float* src = dq_part + (((int64_t)bh * nkb + kb) * RQ + (i - kb * BQ)) * D + c0;
-        const float4 a = *(const float4*)src, c4 = *(const float4*)(src + 4);
-        acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
-        acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
+        const int rel = i - kb * BQ;             // row of the block's reach; segment s holds rel - s*segw in [0, RS)
+        const int s_hi = rel / segw < nseg - 1 ? rel / segw : nseg - 1;
+        const int s_lo = rel - RS + 1 <= 0 ? 0 : (rel - RS + segw) / segw;
+        for (int sg = s_lo; sg <= s_hi; ++sg) {
+            const float* src = dq_part + ((((int64_t)bh * nkb + kb) * nseg + sg) * RS + (rel - sg * segw)) * D + c0;
+            const float4 a = *(const float4*)src, c4 = *(const float4*)(src + 4);
+            acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
+            acc[4] += c4.x; acc[5] += c4.y; acc[6] += c4.z; acc[7] += c4.w;
+        }
     }
     union { EL hh[8]; uint4 u; } o;
 #pragma unroll
@@ -812,64 +851,111 @@ __global__ __launch_bounds__(256) void mfma_bwd_dq_sum_kernel(Problem p, const f
     *(uint4*)((uint16_t*)p.dq.p + p.dq.off(b, i, h) + c0) = o.u;
 }
 
-// units per pair and round of the main kernel: two at head_dim 32 and 64 while the doubled P hand-over
-// still leaves room for the dQ accumulator, else one
+// dK' and dV' from the fp32 partial sums of a segmented launch, segments added in their order
+template <class E>
+__global__ __launch_bounds__(256) void kp_sum_kernel(Problem p, int nseg, const float* __restrict__ kpart, int64_t chunks) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= chunks) return;
+    const int D = p.D;
+    const int col = (int)(c % (D / 4));
+    const int64_t rowid = c / (D / 4);
+    const int k = (int)(rowid % p.N);
+    const int bh = (int)(rowid / p.N);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int64_t BH = (int64_t)p.B * p.H;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const Tensor& t = which ? p.dk2 : p.dv2;
+        if (!t.p) continue;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int sg = 0; sg < nseg; ++sg) {
+            const float4 y = *(const float4*)(kpart + (((which * (int64_t)nseg + sg) * BH + bh) * p.N + k) * D + col * 4);
+            acc.x += y.x; acc.y += y.y; acc.z += y.z; acc.w += y.w;
+        }
+        *(uint2*)((uint16_t*)t.p + t.off(b, k, h) + col * 4) = make_uint2(E::pack(acc.x, acc.y), E::pack(acc.z, acc.w));
+    }
+}
+
+// Geometry of a launch: deltas per segment and number of segments (one while the dQ accumulator of the
+// whole K' window fits LDS).  A pair holds two deltas per round at head_dim 32 and 64, one at 128.
+struct KpPlan {
+    int segw, nseg;
+};
 template <int D>
 constexpr int kp_units() { return D <= 64 ? 2 : 1; }
+template <int D>
+KpPlan kp_plan_of(int w2) {
+    using C = KpCfg<D, kp_units<D>()>;
+    if (C::fits(w2)) return KpPlan{w2 + 1, 1};
+    constexpr int UPR = NPAIR * kp_units<D>();
+    int segw = UPR;
+    while (C::fits(segw + UPR - 1)) segw += UPR;           // whole rounds per segment
+    return KpPlan{segw, (w2 + segw) / segw};
+}
+KpPlan kp_plan(int D, int w2) { return D == 128 ? kp_plan_of<128>(w2) : D == 64 ? kp_plan_of<64>(w2) : kp_plan_of<32>(w2); }
 
-template <class E, int D, int U>
-int launch_kp_units(const Problem& p, hipStream_t st) {
+size_t kp_dq_part_bytes(int B, int N, int H, int D, const KpPlan& pl) {
+    const size_t nkb = (size_t)(N + BQ - 1) / BQ;
+    return ((size_t)B * H * nkb * pl.nseg * (size_t)(BQ + pl.segw - 1) * D * sizeof(float) + 255) / 256 * 256;
+}
+
+template <class E, int D>
+int launch_kp(const Problem& p, hipStream_t st) {
+    constexpr int U = kp_units<D>();
     using C = KpCfg<D, U>;
+    const KpPlan pl = kp_plan(D, p.w2);
     const int nkb = (p.N + BQ - 1) / BQ;
-    const int64_t total = (int64_t)nkb * p.B * p.H;
+    const int64_t total = (int64_t)nkb * p.B * p.H * pl.nseg;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-    if (p.dq.p && p.scratch_bytes < kp_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
-    const bool raw = C::raw_fits(p.w2);
-    const size_t lds = C::lds_bytes(p.w2, raw);
+    if ((p.dq.p || pl.nseg > 1) && p.scratch_bytes < kp_scratch_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+    const int w2s = pl.segw - 1;
+    const bool raw = pl.nseg == 1 && C::raw_fits(w2s);
+    const size_t lds = C::lds_bytes(w2s, raw);
     float* part = (float*)p.scratch;
+    float* kpart = (float*)((char*)p.scratch + kp_dq_part_bytes(p.B, p.N, p.H, D, pl));
     // one unit left over after the rounds of four: the pre-pass takes it
     // (unless the grid is so small that a further launch costs more than the lone round)
-    const int left = (p.w2 >= NPAIR && p.w2 % NPAIR == 0 && (p.force_prepass || total >= 768)) ? 1 : 0;
+    const int left = (pl.nseg == 1 && p.w2 >= NPAIR && p.w2 % NPAIR == 0 && (p.force_prepass || total >= 768)) ? 1 : 0;
     if (left) {
         const size_t lds_left = (size_t)C::NSTAGE * C::STAGE * 2 + KpCfg<D, 1>::PX_BYTES;
         const int ngrp = (nkb + NPAIR - 1) / NPAIR;
         const int64_t total_left = (int64_t)ngrp * p.B * p.H;
         if (!allow_full_lds((const void*)mfma_bwd_kp_kernel<E, D, false, true, 1>)) return SA2_ERR_LAUNCH_FAILED;
         hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, true, 1>), dim3((unsigned)total_left), dim3(KT), lds_left, st, p, ngrp,
-                           (int)total_left, part, 0);
+                           (int)total_left, part, 0, 1, p.w2 + 1, (float*)nullptr);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
-    const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<E, D, true, false, U> : (const void*)mfma_bwd_kp_kernel<E, D, false, false, U>;
-    if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
-    if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, true, false, U>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
-    else hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false, U>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left);
+    if (pl.nseg > 1) {
+        if (!allow_full_lds((const void*)mfma_bwd_kp_kernel<E, D, false, false, U, true>)) return SA2_ERR_LAUNCH_FAILED;
+        hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false, U, true>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb,
+                           (int)total, part, left, pl.nseg, pl.segw, kpart);
+    } else {
+        const void* fn = raw ? (const void*)mfma_bwd_kp_kernel<E, D, true, false, U> : (const void*)mfma_bwd_kp_kernel<E, D, false, false, U>;
+        if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
+        if (raw) hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, true, false, U>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left, 1, p.w2 + 1, kpart);
+        else hipLaunchKernelGGL((mfma_bwd_kp_kernel<E, D, false, false, U>), dim3((unsigned)total), dim3(KT), lds, st, p, nkb, (int)total, part, left, 1, p.w2 + 1, kpart);
+    }
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (p.dq.p) {
         const int64_t items = (int64_t)p.B * p.H * p.N * (D / 8);
         hipLaunchKernelGGL((mfma_bwd_dq_sum_kernel<E, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p, part,
-                           nkb, items);
+                           nkb, items, pl.nseg, pl.segw);
+        if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
+    }
+    if (pl.nseg > 1 && (p.dk2.p || p.dv2.p)) {
+        const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
+        hipLaunchKernelGGL((kp_sum_kernel<E>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, p, pl.nseg, kpart, chunks);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     }
     return SA2_OK;
 }
 
-template <class E, int D>
-int launch_kp(const Problem& p, hipStream_t st) {
-    if constexpr (kp_units<D>() == 2) {
-        if (KpCfg<D, 2>::fits(p.w2)) return launch_kp_units<E, D, 2>(p, st);
-    }
-    return launch_kp_units<E, D, 1>(p, st);
-}
-
 }  // namespace
 
-bool kp_fits(int D, int w2) {
-    return D == 128 ? KpCfg<128, 1>::fits(w2) : D == 64 ? KpCfg<64, 1>::fits(w2) : D == 32 ? KpCfg<32, 1>::fits(w2) : false;
-}
-
+// workspace of the K'-side kernel: the dQ partials, then (segmented launches) the dK' and dV' partials
 size_t kp_scratch_bytes(int B, int N, int H, int D, int w2) {
-    const size_t nkb = (size_t)(N + BQ - 1) / BQ;
-    return (size_t)B * H * nkb * (size_t)(BQ + w2) * D * sizeof(float);
+    const KpPlan pl = kp_plan(D, w2);
+    return kp_dq_part_bytes(B, N, H, D, pl) + (pl.nseg > 1 ? (size_t)2 * pl.nseg * B * H * (size_t)N * D * sizeof(float) : 0);
 }
 
 int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st) {

@@ -54,26 +54,34 @@ struct KvCfg {
         return (size_t)NUNIT * UNIT_BYTES + PX_BYTES + 2 * BQ * FS * 4 + 2 * (size_t)(BQ + w2) * RS * 2 + 4 * BQ * 4;
     }
     static bool fits(int w2) { return lds_bytes(w2) <= LDS_LIMIT; }
+    // widest run of deltas (minus one) whose K'/V' rows LDS holds at once
+    static int max_segment() {
+        return (int)((LDS_LIMIT - lds_bytes(0)) / (2 * (size_t)RS * 2));
+    }
 };
 
 // BIAS = false: k2_bias and v2_bias are both zero (the reference's default), the adds drop out.
 // nsplit > 1: the workgroup takes the sp-th share of the key block's query blocks and writes fp32
 // partial sums to `part` ([2][nsplit][B*H][N][D]: dK before its scale, then dV).
-template <class E, int D, bool BIAS, int KB>
+// SEG = true: a K' window too wide for LDS is walked in segments of ws_arg + 1 deltas; LDS holds the K'/V'
+// rows of one segment of a query block and they are reloaded at every segment.  (A kernel of its own, so that
+// the common case carries none of it.)
+template <class E, int D, bool BIAS, int KB, bool SEG>
 __global__ __launch_bounds__(VT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __restrict__ part) {
+void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __restrict__ part, int ws_arg) {
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
     using C = KvCfg<D, KB>;
     constexpr int VJ = C::VJ;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.N, w1 = p.w1, w2 = p.w2;
-    const int SR = BQ + w2;                                   // K'/V' rows kept per query block
+    const int ws = SEG ? ws_arg : w2;
+    const int SR = BQ + ws;                                   // K'/V' rows kept per query block and segment
     unsigned char* units = smem_raw;
     unsigned char* px = smem_raw + (size_t)C::NUNIT * C::UNIT_BYTES;
     float* q_s = (float*)(px + C::PX_BYTES);                  // [BQ][FS] q * scale*log2(e), fp32
     float* do_s = q_s + BQ * C::FS;                           // [BQ][FS] dO, fp32
-    uint16_t* k2_s = (uint16_t*)(do_s + BQ * C::FS);          // [SR][RS] rows i0-w2 .. i0+31
+    uint16_t* k2_s = (uint16_t*)(do_s + BQ * C::FS);          // [SR][RS] rows i0-dbase-ws .. i0-dbase+31
     uint16_t* v2_s = k2_s + SR * C::RS;                       // [SR][RS]
     float* lse_s = (float*)(v2_s + SR * C::RS);               // [2][BQ]  -LSE*log2(e), by parity of ib
     float* dsum_s = lse_s + 2 * BQ;                           // [2][BQ]  -D_i
@@ -131,7 +139,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
     };
 
     // ---- raw rows of a query block: q, dO, the K'/V' rows its deltas reach, -LSE, -D ----
-    auto load_raw = [&](int ib) {
+    auto load_raw = [&](int ib, int dbase) {
         constexpr int CPR = D / 8;
         const int i0 = ib * BQ;
         for (int c = tid; c < BQ * CPR; c += VT) {
@@ -149,7 +157,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
         }
         for (int c = tid; c < SR * CPR; c += VT) {
             const int row = c / CPR, col = c - row * CPR;
-            int k = i0 - w2 + row;
+            int k = i0 - dbase - ws + row;
             k = k < 0 ? 0 : (k < N ? k : N - 1);
             *(uint4*)(k2_s + row * C::RS + col * 8) = *(const uint4*)(k2p + (int64_t)k * p.k2.sn + col * 8);
             *(uint4*)(v2_s + row * C::RS + col * 8) = *(const uint4*)(v2p + (int64_t)k * p.v2.sn + col * 8);
@@ -178,10 +186,10 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
         qv[0] = q0.x; qv[1] = q0.y; qv[2] = q0.z; qv[3] = q0.w; qv[4] = q1.x; qv[5] = q1.y; qv[6] = q1.z; qv[7] = q1.w;
         dv[0] = d0.x; dv[1] = d0.y; dv[2] = d0.z; dv[3] = d0.w; dv[4] = d1.x; dv[5] = d1.y; dv[6] = d1.z; dv[7] = d1.w;
     };
-    auto form = [&](int delta, int slot) {
+    auto form = [&](int dseg, int slot) {        // dseg: delta - first delta of its segment
         if (!former) return;
         const int row = f_row, col = f_col;
-        const int kr = row - delta + w2;
+        const int kr = row - dseg + ws;
         const uint4 kx = *(const uint4*)(k2_s + kr * C::RS + col * 8);
         const uint4 vx = *(const uint4*)(v2_s + kr * C::RS + col * 8);
         const uint32_t kw[4] = {kx.x, kx.y, kx.z, kx.w}, vw[4] = {vx.x, vx.y, vx.z, vx.w};
@@ -216,7 +224,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
 
     // ---- prologue: first block's raw rows, first unit --------------------------------
     if (has_work) {
-        load_raw(ib_lo);
+        load_raw(ib_lo, 0);
         __syncthreads();
         fetch_qd();
         form(0, 0);
@@ -226,7 +234,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
     // The sweep, instantiated once per role so that each keeps only its own registers live.
     auto sweep = [&](auto role_tag) {
         constexpr int ROLE = decltype(role_tag)::value;
-        int ib = ib_lo, delta = 0, slot = 0, step = 0;
+        int ib = ib_lo, delta = 0, slot = 0, step = 0, dbase = 0;
         int nu = units_of(ib_lo);
         int cur_ib = -1;
         floatx16 negr;                               // -LSE*log2e (P) or -D (dS) of the block's rows, per accumulator element
@@ -388,14 +396,15 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
             const bool more = nib <= ib_hi;
             const int nslot = slot + 1 == C::NUNIT ? 0 : slot + 1;
             if (more) {
-                if (nib != ib) {
+                if (nib != ib || (SEG && ndelta - dbase > ws)) {
+                    if constexpr (SEG) dbase = ndelta;
                     __syncthreads();         // nobody still forms from the old rows
-                    load_raw(nib);
+                    load_raw(nib, dbase);
                     __syncthreads();
                     fetch_qd();
                     nu = units_of(nib);
                 }
-                form(ndelta, nslot);
+                form(ndelta - dbase, nslot);
             }
             __syncthreads();
             ++step;
@@ -495,7 +504,8 @@ int launch_kv_geometry(const Problem& p, int nsplit, hipStream_t st) {
     const int njb = (p.N + C::VJ - 1) / C::VJ;
     const int64_t total = (int64_t)njb * p.B * p.H * nsplit;
     if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
-    const size_t lds = C::lds_bytes(p.w2);
+    const int ws = p.w2 < C::max_segment() ? p.w2 : C::max_segment();
+    const size_t lds = C::lds_bytes(ws);
     const bool bias = p.k2_bias != 0.f || p.v2_bias != 0.f;
     // the partial sums of a split launch lie behind the K'-side kernel's part of the workspace
     float* part = nullptr;
@@ -504,10 +514,15 @@ int launch_kv_geometry(const Problem& p, int nsplit, hipStream_t st) {
         if (p.scratch_bytes < off + kv_split_scratch_bytes(p.B, p.N, p.H, D, p.w1)) return SA2_ERR_WORKSPACE_TOO_SMALL;
         part = (float*)((char*)p.scratch + off);
     }
-    const void* fn = bias ? (const void*)mfma_bwd_kv_kernel<E, D, true, KB> : (const void*)mfma_bwd_kv_kernel<E, D, false, KB>;
+    const bool seg = ws < p.w2;
+    // (the segmented kernel exists with the bias adds only)
+    const void* fn = seg    ? (const void*)mfma_bwd_kv_kernel<E, D, true, KB, true>
+                     : bias ? (const void*)mfma_bwd_kv_kernel<E, D, true, KB, false>
+                            : (const void*)mfma_bwd_kv_kernel<E, D, false, KB, false>;
     if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
-    if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true, KB>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part);
-    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false, KB>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part);
+    if (seg) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true, KB, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
+    else if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true, KB, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
+    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false, KB, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (nsplit > 1) {
         const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
@@ -527,11 +542,6 @@ int launch_kv(const Problem& p, hipStream_t st) {
 }
 
 }  // namespace
-
-bool kv_fits(int D, int w2) {
-    // (two K blocks per pair need the larger hand-over buffer: the limit is theirs at head_dim 64)
-    return D == 128 ? KvCfg<128, 1>::fits(w2) : D == 64 ? KvCfg<64, 2>::fits(w2) : D == 32 ? KvCfg<32, 1>::fits(w2) : false;
-}
 
 size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1) {
     const KvPlan pl = kv_plan(B, N, H, D, w1);

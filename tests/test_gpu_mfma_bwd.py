@@ -29,15 +29,18 @@ SMALL = [  # B, N, H, D, w1, w2, k2_bias, v2_bias
     (1, 1, 1, 64, 4, 4, 0.0, 0.0),
     (2, 130, 2, 32, 33, 8, 0.1, 0.2),         # head_dim 32
     (1, 200, 1, 32, 64, 32, 0.0, 0.0),
-    (1, 200, 1, 128, 16, 150, 0.0, 0.1),     # K' window too wide for the on-chip kernels: workspace kernels
-    (1, 180, 2, 128, 40, 100, 0.2, 0.0),     # K'-side on chip (q, dO rows from global memory), K-side workspace kernel
-    (1, 150, 1, 128, 20, 65, 0.0, 0.0),      # first K' window beyond the K-side on-chip kernel (64 is its last)
-    (1, 190, 1, 128, 12, 113, 0.0, 0.0),     # last K' window of the K'-side on-chip kernel
-    (1, 190, 1, 128, 12, 114, 0.0, 0.0),     # first one beyond it
-    (1, 350, 1, 64, 12, 304, 0.0, 0.0),      # head_dim 64: last K' window with two deltas per wavefront pair
-    (1, 350, 1, 64, 12, 305, 0.1, 0.0),      # first with one delta per pair
-    (1, 390, 1, 64, 9, 362, 0.0, 0.0),       # last K' window of the K'-side on-chip kernel at head_dim 64
-    (1, 390, 1, 64, 9, 363, 0.0, 0.0),       # first one beyond it
+    (1, 200, 1, 128, 16, 150, 0.0, 0.1),     # K' window wider than both kernels' LDS buffers: walked in segments of deltas
+    (1, 180, 2, 128, 40, 100, 0.2, 0.0),     # K'-side in one piece (q, dO rows from global memory), K-side in segments
+    (1, 150, 1, 128, 20, 65, 0.0, 0.0),      # first K' window the K-side kernel walks in two segments (64 is the last in one)
+    (1, 190, 1, 128, 12, 113, 0.0, 0.0),     # last K' window the K'-side kernel takes in one segment
+    (1, 190, 1, 128, 12, 114, 0.0, 0.0),     # first one in two
+    (1, 350, 1, 64, 12, 304, 0.0, 0.0),      # head_dim 64: last K' window of one segment
+    (1, 350, 1, 64, 12, 305, 0.1, 0.0),      # first of two (the second holds one delta)
+    (1, 390, 1, 64, 9, 362, 0.0, 0.0),
+    (2, 300, 2, 128, 16, 230, 0.1, -0.2),    # three segments (112, 112, 7 deltas), several heads
+    (1, 100, 1, 128, 16, 300, 0.0, 0.0),     # window wider than the sequence: the later segments are empty
+    (1, 700, 1, 64, 20, 650, 0.0, 0.0),      # head_dim 64, three segments
+    (1, 900, 1, 32, 8, 850, 0.0, 0.1),       # head_dim 32, both kernels in two segments
 ]
 
 
@@ -58,10 +61,10 @@ def test_small_shapes_vs_oracle(case):
 
 
 @pytest.mark.parametrize("case", [SMALL[1], SMALL[6], (1, 300, 2, 64, 96, 16, 0.1, 0.0), (2, 160, 2, 128, 64, 33, 0.0, 0.0),
-                                  SMALL[12], SMALL[13],                  # workspace kernels
+                                  SMALL[12], SMALL[13],                  # K' windows in segments
                                   (1, 400, 1, 64, 24, 330, 0.0, 0.1)])   # the same at head_dim 64
 def test_small_shapes_fp16_vs_oracle(case):
-    """fp16 elements on the same kernels (fp16 MFMA), the workspace kernels for wide K' windows included.
+    """fp16 elements on the same kernels (fp16 MFMA), K' windows walked in segments included.
     Tolerance: max|diff| <= 1.5e-2 * max|ref| per tensor.  The products q*k2~ and dO*v2~ are rounded to
     fp16 before the MFMAs, as the reference rounds its products to the GEMM type (kernels.py:106,
     301-302); over most of a tensor that costs 1e-3, but on the first query rows, whose windows hold
@@ -181,6 +184,34 @@ def test_needs_input_grad_subsets_and_determinism():
                 assert torch.equal(leaves[t].grad, full[name]), name
             else:
                 assert leaves[t].grad is None
+
+
+def test_segmented_k2_windows_half_open_subsets_and_determinism():
+    """A K' window that both backward kernels walk in segments (head_dim 128, w2 = 180: 112 + 69 deltas on the
+    K'-side, 65 + 65 + 51 on the K-side): the half-open window convention against the oracle, bitwise repeatability,
+    and the gradient subsets of needs_input_grad bit for bit."""
+    import simplical_attn_amd as sa
+    dev = torch.device("cuda:0")
+    inp = make_inputs(1, 260, 2, 128, seed=5, dtype=torch.bfloat16)
+    w1, w2 = 30, 180
+    got = run_device(inp, w1, w2, None, 0.1, 0.0, flags=MFMA, inclusive=False)
+    want = oracle_all(inp, w1, w2, None, 0.1, 0.0, inclusive=False)
+    for name in GRADS:
+        assert_close_rel(got[name], want[name], BF16_TOL, name + " half-open, segments")
+    x = [t.to(dev) for t in inp]
+    out, lse = sa.simplicial_forward(*x[:5], w1, w2, flags=MFMA)
+    full = sa.simplicial_backward(*x[:5], out, lse, x[5], w1, w2, flags=MFMA)
+    again = sa.simplicial_backward(*x[:5], out, lse, x[5], w1, w2, flags=MFMA)
+    for name, a, b in zip(GRADS, full, again):
+        assert torch.equal(a, b), name
+    for subset in ((0,), (1, 3), (2, 4), (2,)):
+        needs = tuple(t in subset for t in range(5))
+        part = sa.simplicial_backward(*x[:5], out, lse, x[5], w1, w2, needs=needs, flags=MFMA)
+        for t, name in enumerate(GRADS):
+            if t in subset:
+                assert torch.equal(part[t], full[t]), name
+            else:
+                assert part[t] is None
 
 
 def test_headline_shape_scaling_and_swap_properties():
