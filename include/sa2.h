@@ -67,10 +67,9 @@ int sa2_version(void);
 const char* sa2_strerror(int status);
 
 /* 1 if sa2_forward would take MFMA kernels for this problem under SA2_FLAG_AUTO
- * (given 16-byte aligned rows), 0 if it would take the fp32-FMA kernels.  It answers for
- * the forward only: sa2_backward additionally falls back to the fp32-FMA kernels when the K' window
- * exceeds what its on-chip accumulators hold (16-bit D = 256: w2 > 82; fp32: w2 > 86, 378, 913 at
- * D = 128, 64, 32; the 16-bit kernels for D = 32, 64, 128 take any window). */
+ * (given 16-byte aligned rows), 0 if it would take the fp32-FMA kernels.  sa2_backward makes the
+ * same choice: its MFMA kernels take any K' window (one wider than their on-chip accumulators hold
+ * is walked in segments of deltas). */
 int sa2_uses_mfma(int B, int N, int H, int D, int w1, int w2, int dtype);
 
 /*

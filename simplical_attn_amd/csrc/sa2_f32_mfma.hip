@@ -49,6 +49,14 @@ struct F32Cfg {
     // K'-side kernel: the stages, the dQ accumulator (32 + w2 rows) and the dK' and dV' accumulators (32 rows each)
     static size_t kp_lds(int w2) { return TILES_BYTES + (size_t)(32 + w2 + 64) * RS * 4; }
     static bool kp_fits(int w2) { return kp_lds(w2) <= LDS_LIMIT; }
+    // deltas whose dQ rows the accumulator holds at once: all w2 + 1 of them, or (wider K' windows) the largest
+    // multiple of four that fits; the kernel then walks the window in segments of that many deltas
+    static int kp_segment(int w2) {
+        if (kp_fits(w2)) return w2 + 1;
+        int segw = 32;
+        while (kp_fits(segw + XW - 1)) segw += XW;
+        return segw;
+    }
     static constexpr size_t KV_LDS = TILES_BYTES + 2 * 2 * 32 * 4;
 };
 
@@ -297,14 +305,15 @@ void f32_fwd_kernel(Problem p, int nqb, int total) {
 }
 
 // ============================================== backward, K' side: dQ, dK', dV' =====
-template <int D>
+// SEG: the K' window is walked in segments of segw deltas (a kernel of its own; segw = w2 + 1 otherwise)
+template <int D, bool SEG>
 __global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) {
+void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int segw) {
     using C = F32Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) float smem_f[];
     float* dk_s = smem_f + 2 * C::STAGE;         // [32][RS]: dK' rows k0 .. k0+31 (before the scale)
     float* dv_s = dk_s + 32 * C::RS;             // [32][RS]: dV' rows
-    float* dq_s = dv_s + 32 * C::RS;             // [32 + w2][RS]: dQ rows k0 .. k0+31+w2 (before the scale)
+    float* dq_s = dv_s + 32 * C::RS;             // [32 + segw - 1][RS]: dQ rows k0 + dbase .. of the current segment (before the scale)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -314,7 +323,9 @@ void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_par
     const int b = bh / p.H, h = bh - b * p.H;
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int k0 = kb * BQ, k = k0 + ln, kc = k < N ? k : N - 1;
-    const int NR = 32 + w2;
+    const int NR = 32 + w2;                      // rows of the block's dQ partial
+    const int NRS = 32 + segw - 1;               // rows of the accumulator
+    int dbase = 0;                               // first delta of the current segment
 
     const float* qp = (const float*)p.q.p + p.q.off(b, 0, h);
     const float* k1p = (const float*)p.k1.p + p.k1.off(b, 0, h);
@@ -328,7 +339,7 @@ void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_par
     const int nrounds = (n_units + XW - 1) / XW;
     const float qscale = p.scale * LOG2E;
 
-    for (int c = tid; c < (NR + 64) * C::RS; c += XT) dk_s[c] = 0.f;       // all three accumulators
+    for (int c = tid; c < (NRS + 64) * C::RS; c += XT) dk_s[c] = 0.f;      // all three accumulators
 
     fx4 tk[C::KR], tv[C::KR];                    // the tile on its way from global memory to LDS
     for (int round = 0; round < nrounds; ++round) {
@@ -434,7 +445,7 @@ void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_par
                 const float* krow = k2p + (int64_t)kc * p.k2.sn + col;
                 float* dkrow = dk_s + ln * C::RS + col;
                 float* dvrow = dv_s + ln * C::RS + col;
-                float* dqrow = dq_s + (ln + delta) * C::RS + col;
+                float* dqrow = dq_s + (ln + delta - dbase) * C::RS + col;
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt) {
                     // (g4 is uniform over the wavefront: pick this group's four registers)
@@ -463,6 +474,29 @@ void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_par
             }
             __syncthreads();
         }
+        // ---- end of a segment: its first segw dQ rows are complete and go to the partial; the 31 rows the next
+        //      segment shares with it move to the front of the accumulator ----
+        if (SEG && round + 1 < nrounds && (round + 1) * XW - dbase >= segw) {
+            if (want_dq) {
+                float* part = dq_part + (((int64_t)bh * nkb + kb) * (int64_t)NR + dbase) * D;
+                for (int c = tid; c < segw * (D / 4); c += XT) {
+                    const int r = c / (D / 4), col = c - r * (D / 4);
+                    *(float4*)(part + (int64_t)r * D + col * 4) = *(const float4*)(dq_s + r * C::RS + col * 4);
+                }
+                __syncthreads();
+                for (int c = tid; c < 31 * (D / 4); c += XT) {          // (segw >= 32: source and destination are disjoint)
+                    const int r = c / (D / 4), col = c - r * (D / 4);
+                    *(float4*)(dq_s + r * C::RS + col * 4) = *(const float4*)(dq_s + (segw + r) * C::RS + col * 4);
+                }
+                __syncthreads();
+                for (int c = tid; c < (NRS - 31) * (D / 4); c += XT) {
+                    const int r = 31 + c / (D / 4), col = c % (D / 4);
+                    *(float4*)(dq_s + r * C::RS + col * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+                __syncthreads();
+            }
+            dbase += segw;
+        }
     }
 
     // ---- dK' and dV' rows of the block ----
@@ -481,12 +515,14 @@ void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_par
             }
         }
     }
-    // ---- dQ partial of this block: rows k0 .. k0+31+w2 ----
+    // ---- dQ partial of this block: rows k0 .. k0+31+w2, of which those from dbase on are still here
+    //      (rows past the accumulator belong to deltas beyond the end of the sequence: zeros) ----
     if (want_dq) {
-        float* part = dq_part + ((int64_t)bh * nkb + kb) * (int64_t)NR * D;
-        for (int c = tid; c < NR * (D / 4); c += XT) {
+        float* part = dq_part + (((int64_t)bh * nkb + kb) * (int64_t)NR + dbase) * D;
+        for (int c = tid; c < (NR - dbase) * (D / 4); c += XT) {
             const int r = c / (D / 4), col = c - r * (D / 4);
-            *(float4*)(part + (int64_t)r * D + col * 4) = *(const float4*)(dq_s + r * C::RS + col * 4);
+            *(float4*)(part + (int64_t)r * D + col * 4) =
+                r < NRS ? *(const float4*)(dq_s + r * C::RS + col * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
 }
@@ -766,8 +802,13 @@ int launch_f32_bwd(const Problem& p, hipStream_t st) {
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
         if (p.scratch_bytes < f32_dq_part_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
         float* part = (float*)p.scratch;
-        if (!allow_full_lds((const void*)f32_bwd_kp_kernel<D>)) return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL((f32_bwd_kp_kernel<D>), dim3((unsigned)total), dim3(XT), C::kp_lds(p.w2), st, p, nkb, (int)total, part);
+        const int segw = C::kp_segment(p.w2);
+        if (!allow_full_lds((const void*)f32_bwd_kp_kernel<D, false>) || !allow_full_lds((const void*)f32_bwd_kp_kernel<D, true>))
+            return SA2_ERR_LAUNCH_FAILED;
+        if (segw < p.w2 + 1)
+            hipLaunchKernelGGL((f32_bwd_kp_kernel<D, true>), dim3((unsigned)total), dim3(XT), C::kp_lds(segw - 1), st, p, nkb, (int)total, part, segw);
+        else
+            hipLaunchKernelGGL((f32_bwd_kp_kernel<D, false>), dim3((unsigned)total), dim3(XT), C::kp_lds(segw - 1), st, p, nkb, (int)total, part, segw);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
         if (p.dq.p) {
             const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
@@ -812,8 +853,8 @@ bool rows16(const Tensor& t, int B, int N, int H) {
 bool f32_mfma_supported(int D, int dtype) { return dtype == SA2_F32 && (D == 32 || D == 64 || D == 128); }
 
 bool f32_mfma_bwd_supported(int D, int w2, int dtype) {
-    if (!f32_mfma_supported(D, dtype)) return false;
-    return D == 128 ? F32Cfg<128>::kp_fits(w2) : D == 64 ? F32Cfg<64>::kp_fits(w2) : F32Cfg<32>::kp_fits(w2);
+    (void)w2;                // any K' window: wide ones are walked in segments
+    return f32_mfma_supported(D, dtype);
 }
 
 bool f32_mfma_layout_ok(const Problem& p, bool backward) {

@@ -53,6 +53,14 @@ struct WideCfg {
     static constexpr size_t LDS_LIMIT = 160 * 1024;
     static size_t kp_lds(int w2) { return TILES_BYTES + (size_t)(32 + w2 + 64) * AS * 4; }
     static bool kp_fits(int w2) { return kp_lds(w2) <= LDS_LIMIT; }
+    // deltas whose dQ rows the accumulator holds at once: all w2 + 1 of them, or (wider K' windows) the largest
+    // multiple of four that fits; the kernel then walks the window in segments of that many deltas
+    static int kp_segment(int w2) {
+        if (kp_fits(w2)) return w2 + 1;
+        int segw = 32;
+        while (kp_fits(segw + WW - 1)) segw += WW;
+        return segw;
+    }
     static constexpr size_t KV_LDS = TILES_BYTES + 2 * 2 * 32 * 4;
 };
 
@@ -332,9 +340,10 @@ void wide_fwd_kernel(Problem p, int nqb, int total) {
 }
 
 // ============================================== backward, K' side: dQ, dK', dV' =====
-template <class E, int D, int DV>
+// SEG: the K' window is walked in segments of segw deltas (a kernel of its own; segw = w2 + 1 otherwise)
+template <class E, int D, int DV, bool SEG>
 __global__ __launch_bounds__(WT) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) {
+void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int segw) {
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
     using C = WideCfg<D, DV>;
@@ -342,7 +351,7 @@ void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) 
     uint16_t* tiles = (uint16_t*)smem_w;
     float* dk_s = (float*)(smem_w + C::TILES_BYTES);     // [32][AS]: dK' rows k0 .. k0+31 (before the scale)
     float* dv_s = dk_s + 32 * C::AS;                     // [32][AS]: dV' rows
-    float* dq_s = dv_s + 32 * C::AS;                     // [32 + w2][AS]: dQ rows k0 .. k0+31+w2 (before the scale)
+    float* dq_s = dv_s + 32 * C::AS;                     // [32 + segw - 1][AS]: dQ rows k0 + dbase .. of the current segment (before the scale)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -353,7 +362,9 @@ void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) 
     const int b = bh / p.H, h = bh - b * p.H;
     const int N = p.N, w1 = p.w1, w2 = p.w2;
     const int k0 = kb * BQ, k = k0 + ln, kc = k < N ? k : N - 1;
-    const int NR = 32 + w2;
+    const int NR = 32 + w2;                      // rows of the block's dQ partial
+    const int NRS = 32 + segw - 1;               // rows of the accumulator
+    int dbase = 0;                               // first delta of the current segment
 
     const uint16_t* qp = (const uint16_t*)p.q.p + p.q.off(b, 0, h);
     const uint16_t* k1p = (const uint16_t*)p.k1.p + p.k1.off(b, 0, h);
@@ -369,7 +380,7 @@ void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) 
     const uint32_t tiles_addr = lds_address(tiles);
     const uint32_t tr_lane = tr_lane_offset<C::RSB>(lane);
 
-    for (int c = tid; c < (NR + 64) * C::AS; c += WT) dk_s[c] = 0.f;       // all three accumulators
+    for (int c = tid; c < (NRS + 64) * C::AS; c += WT) dk_s[c] = 0.f;      // all three accumulators
 
     ux4 tk[C::KR], tv[C::KR];
     for (int round = 0; round < nrounds; ++round) {
@@ -466,7 +477,7 @@ void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) 
                 const uint16_t* krow = k2p + (int64_t)kc * p.k2.sn + c0 + col;
                 float* dkrow = dk_s + ln * C::AS + col;
                 float* dvrow = dv_s + ln * C::AS + col;
-                float* dqrow = dq_s + (ln + delta) * C::AS + col;
+                float* dqrow = dq_s + (ln + delta - dbase) * C::AS + col;
 #pragma unroll
                 for (int dt = 0; dt < C::DT; ++dt) {
                     // (g4 is uniform over the wavefront: pick this group's four registers)
@@ -495,6 +506,29 @@ void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) 
             }
             __syncthreads();
         }
+        // ---- end of a segment: its first segw dQ rows are complete and go to the partial; the 31 rows the next
+        //      segment shares with it move to the front of the accumulator ----
+        if (SEG && round + 1 < nrounds && (round + 1) * WW - dbase >= segw) {
+            if (want_dq) {
+                float* part = dq_part + (((int64_t)bh * nkb + kb) * (int64_t)NR + dbase) * D + c0;
+                for (int c = tid; c < segw * (DV / 4); c += WT) {
+                    const int r = c / (DV / 4), col = c - r * (DV / 4);
+                    *(float4*)(part + (int64_t)r * D + col * 4) = *(const float4*)(dq_s + r * C::AS + col * 4);
+                }
+                __syncthreads();
+                for (int c = tid; c < 31 * (DV / 4); c += WT) {         // (segw >= 32: source and destination are disjoint)
+                    const int r = c / (DV / 4), col = c - r * (DV / 4);
+                    *(float4*)(dq_s + r * C::AS + col * 4) = *(const float4*)(dq_s + (segw + r) * C::AS + col * 4);
+                }
+                __syncthreads();
+                for (int c = tid; c < (NRS - 31) * (DV / 4); c += WT) {
+                    const int r = 31 + c / (DV / 4), col = c % (DV / 4);
+                    *(float4*)(dq_s + r * C::AS + col * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+                __syncthreads();
+            }
+            dbase += segw;
+        }
     }
 
     // ---- dK' and dV' rows of the block (this pass's columns) ----
@@ -517,11 +551,14 @@ void wide_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part) 
         }
     }
     // ---- dQ partial of this block: rows k0 .. k0+31+w2, this pass's columns ----
+    //      (those from dbase on are still here; rows past the accumulator belong to deltas beyond the end of the
+    //      sequence: zeros)
     if (want_dq) {
-        float* part = dq_part + ((int64_t)bh * nkb + kb) * (int64_t)NR * D + c0;
-        for (int c = tid; c < NR * (DV / 4); c += WT) {
+        float* part = dq_part + (((int64_t)bh * nkb + kb) * (int64_t)NR + dbase) * D + c0;
+        for (int c = tid; c < (NR - dbase) * (DV / 4); c += WT) {
             const int r = c / (DV / 4), col = c - r * (DV / 4);
-            *(float4*)(part + (int64_t)r * D + col * 4) = *(const float4*)(dq_s + r * C::AS + col * 4);
+            *(float4*)(part + (int64_t)r * D + col * 4) =
+                r < NRS ? *(const float4*)(dq_s + r * C::AS + col * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
 }
@@ -805,9 +842,15 @@ int launch_wide_bwd(const Problem& p, hipStream_t st) {
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
         if (p.scratch_bytes < wide_dq_part_bytes(p.B, p.N, p.H, D, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
         float* part = (float*)p.scratch;
-        if (!allow_full_lds((const void*)wide_kp_kernel<E, D, DV>)) return SA2_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL((wide_kp_kernel<E, D, DV>), dim3((unsigned)total, C::NPASS), dim3(WT), C::kp_lds(p.w2), st, p, nkb, (int)total,
-                           part);
+        if (!allow_full_lds((const void*)wide_kp_kernel<E, D, DV, false>) || !allow_full_lds((const void*)wide_kp_kernel<E, D, DV, true>))
+            return SA2_ERR_LAUNCH_FAILED;
+        const int segw = C::kp_segment(p.w2);
+        if (segw < p.w2 + 1)
+            hipLaunchKernelGGL((wide_kp_kernel<E, D, DV, true>), dim3((unsigned)total, C::NPASS), dim3(WT), C::kp_lds(segw - 1), st, p, nkb,
+                               (int)total, part, segw);
+        else
+            hipLaunchKernelGGL((wide_kp_kernel<E, D, DV, false>), dim3((unsigned)total, C::NPASS), dim3(WT), C::kp_lds(segw - 1), st, p, nkb,
+                               (int)total, part, segw);
         if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
         if (p.dq.p) {
             const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
@@ -847,7 +890,10 @@ int launch_wide_bwd(const Problem& p, hipStream_t st) {
 
 bool wide_supported(int D, int dtype) { return (dtype == SA2_BF16 || dtype == SA2_F16) && D == 256; }
 
-bool wide_bwd_supported(int D, int w2, int dtype) { return wide_supported(D, dtype) && WideCfg<256, 128>::kp_fits(w2); }
+bool wide_bwd_supported(int D, int w2, int dtype) {
+    (void)w2;                // any K' window: wide ones are walked in segments
+    return wide_supported(D, dtype);
+}
 
 size_t wide_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
     const int ns = wide_kv_nsplit(B, N, H, D, w1, 2);

@@ -190,18 +190,24 @@ def test_unaligned_fp32_rows_take_the_fma_kernels():
         assert_close_rel(a, want[name], 1e-5, name)
 
 
-def test_wide_k2_window_falls_back_in_the_backward_only():
-    """head_dim 128 with a K' window beyond what the K'-side kernel's LDS accumulators hold: the forward
-    still takes the MFMA kernel, the backward the FMA kernels; both match the oracle."""
+@pytest.mark.parametrize("case", [(1, 160, 1, 128, 8, 120, 0.0), (1, 300, 2, 128, 20, 260, 0.2), (1, 500, 1, 64, 6, 450, 0.0),
+                                  (1, 100, 1, 128, 8, 200, 0.0)],
+                         ids=lambda c: "N%d-D%d-w%d_%d" % (c[1], c[3], c[4], c[5]))
+def test_wide_k2_windows_are_walked_in_segments(case):
+    """K' windows beyond what the K'-side kernel's dQ accumulator holds in LDS (86 deltas at head_dim 128, 378 at 64):
+    the kernel walks them in segments of 84 / 376 deltas (two, four and two segments here; in the last case the
+    window is wider than the sequence).  Forced and under the default dispatch (same bits), against the oracle."""
     import simplical_attn_amd as sa
     dev = torch.device("cuda:0")
-    B, N, H, D, w1, w2 = 1, 160, 1, 128, 8, 120
+    B, N, H, D, w1, w2, kb = case
     host = make_inputs(B, N, H, D, seed=12, mag=0.5)
     x = [t.to(dev) for t in host]
-    out, lse = sa.simplicial_forward(*x[:5], w1, w2, flags=MFMA)
-    with pytest.raises(_lib.Sa2Error):
-        sa.simplicial_backward(*x[:5], out, lse, x[5], w1, w2, flags=MFMA)
-    grads = sa.simplicial_backward(*x[:5], out, lse, x[5], w1, w2)
-    want = oracle_all(host, w1, w2)
-    for name, a in zip(NAMES, (out, lse, *grads)):
+    res = {}
+    for flags in (MFMA, AUTO):
+        out, lse = sa.simplicial_forward(*x[:5], w1, w2, None, kb, 0.0, flags=flags)
+        grads = sa.simplicial_backward(*x[:5], out, lse, x[5], w1, w2, None, kb, 0.0, flags=flags)
+        res[flags] = (out, lse, *grads)
+    want = oracle_all(host, w1, w2, None, kb, 0.0)
+    for name, a, b in zip(NAMES, res[MFMA], res[AUTO]):
+        assert torch.equal(a, b), name
         assert_close_rel(a, want[name], 1e-5, name)

@@ -139,20 +139,22 @@ def test_longer_sequence_against_oracle_row_ranges_and_the_fp32_kernels():
         assert_close_rel(got["lse"][:, :, rows[0]:rows[1]], want_lse, 2e-2, "lse rows %s" % (rows,))
 
 
-def test_wide_k2_window_and_unaligned_rows_fall_back():
-    """A K' window beyond the K'-side kernel's LDS accumulators (w2 > 82): forward on MFMA, backward on the
-    fp32 kernels.  Rows off the 16-byte grid: everything on the fp32 kernels.  Both match the oracle."""
+def test_wide_k2_windows_in_segments_and_unaligned_rows():
+    """K' windows beyond the K'-side kernel's dQ accumulator in LDS (w2 > 82) are walked in segments of 80 deltas
+    (two and four segments here), forced and under the default dispatch (same bits), against the oracle.
+    Rows off the 16-byte grid: everything on the fp32 kernels."""
     import simplical_attn_amd as sa
     dev = torch.device("cuda:0")
+    for N, w1, w2, kb in ((160, 8, 120, 0.0), (290, 12, 250, 0.1)):
+        host = make_inputs(1, N, 1, D, seed=12, dtype=torch.bfloat16, mag=0.5)
+        x = [t.to(dev) for t in host]
+        a = _run(sa, x, w1, w2, kb, 0.0, MFMA)
+        b = _run(sa, x, w1, w2, kb, 0.0, AUTO)
+        want = oracle_all(host, w1, w2, None, kb, 0.0)
+        for name in NAMES:
+            assert torch.equal(a[name], b[name]), name
+            assert_close_rel(a[name], want[name], 2e-2, "%s w2=%d" % (name, w2))
     host = make_inputs(1, 160, 1, D, seed=12, dtype=torch.bfloat16, mag=0.5)
-    x = [t.to(dev) for t in host]
-    out, lse = sa.simplicial_forward(*x[:5], 8, 120, flags=MFMA)
-    with pytest.raises(_lib.Sa2Error):
-        sa.simplicial_backward(*x[:5], out, lse, x[5], 8, 120, flags=MFMA)
-    grads = sa.simplicial_backward(*x[:5], out, lse, x[5], 8, 120)
-    want = oracle_all(host, 8, 120)
-    for name, a in zip(NAMES, (out, lse, *grads)):
-        assert_close_rel(a, want[name], 2e-2, name)
     wide = [torch.zeros(1, 160, 1, D + 8, dtype=torch.bfloat16, device=dev) for _ in host]
     views = [w[..., 4:4 + D] for w in wide]
     for v, t in zip(views, host):
