@@ -105,7 +105,7 @@ __device__ __forceinline__ void tile_store(const fx4 (&a)[F32Cfg<D>::KR], const 
 
 // ================================================================== forward =====
 template <int D>
-__global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 2 : 1, D <= 64 ? 2 : 1)))
 void f32_fwd_kernel(Problem p, int nqb, int total) {
     using C = F32Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) float smem_f[];
@@ -307,7 +307,7 @@ void f32_fwd_kernel(Problem p, int nqb, int total) {
 // ============================================== backward, K' side: dQ, dK', dV' =====
 // SEG: the K' window is walked in segments of segw deltas (a kernel of its own; segw = w2 + 1 otherwise)
 template <int D, bool SEG>
-__global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 2 : 1, D <= 64 ? 2 : 1)))
 void f32_bwd_kp_kernel(Problem p, int nkb, int total, float* __restrict__ dq_part, int segw) {
     using C = F32Cfg<D>;
     extern __shared__ __attribute__((aligned(16))) float smem_f[];
@@ -554,7 +554,7 @@ __global__ __launch_bounds__(256) void f32_dq_sum_kernel(Problem p, int nkb, con
 // nsplit > 1 (grids smaller than the chip): the workgroup takes the sp-th share of the key block's query
 // blocks and writes fp32 partial sums to `part` ([dK | dV][nsplit][B*H][N][D]) for f32_kv_sum_kernel.
 template <int D, bool SPLIT>
-__global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 2 : 1, D <= 64 ? 2 : 1)))
 void f32_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __restrict__ part) {
     const int nsplit = SPLIT ? nsplit_arg : 1;
     using C = F32Cfg<D>;
