@@ -12,7 +12,9 @@
 // deltas a wavefront handles; dQ is shifted by delta and goes through an fp32 accumulator
 // in LDS (rows k0 .. k0+31+w2), written once per workgroup as a partial that a small
 // kernel adds up (a query gets partials from at most 2 + w2/32 workgroups, summed in a
-// fixed order: bitwise reproducible).
+// fixed order: bitwise reproducible).  A K' window too wide for that accumulator is cut into
+// segments of deltas, one workgroup per (K' block, segment); their fp32 partial dK' and dV' are
+// added by kp_sum_kernel in segment order.
 //
 // Eight wavefronts, two per SIMD, form four pairs that each hold one unit per round (two
 // consecutive deltas at head_dim 32 and 64, where the registers allow it: every K and V operand
