@@ -105,7 +105,7 @@ int launch_mfma_bwd_kp(const Problem& p, int dtype, hipStream_t st);
 // K-side backward kernel (dK, dV) with paired wavefronts; for small grids it splits a key block's
 // query blocks over several workgroups, whose fp32 partial sums lie in the workspace behind the
 // K'-side part (kp_side_scratch_bytes); K' windows too wide for its LDS rows are walked in segments
-size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1);
+size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1, int w2);
 size_t kp_side_scratch_bytes(int B, int N, int H, int D, int w2);
 int launch_mfma_bwd_kv(const Problem& p, int dtype, hipStream_t st);
 

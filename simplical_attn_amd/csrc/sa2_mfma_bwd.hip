@@ -23,7 +23,7 @@ size_t kp_side_scratch_bytes(int B, int N, int H, int D, int w2) {
 }
 
 size_t mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
-    return kp_side_scratch_bytes(B, N, H, D, w2) + kv_split_scratch_bytes(B, N, H, D, w1);
+    return kp_side_scratch_bytes(B, N, H, D, w2) + kv_split_scratch_bytes(B, N, H, D, w1, w2);
 }
 
 int launch_mfma_bwd(const Problem& p, int dtype, hipStream_t st) {

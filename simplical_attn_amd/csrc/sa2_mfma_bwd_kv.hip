@@ -15,9 +15,9 @@
 // out in row groups so that both kinds of read are free of bank conflicts.
 // Every output element has one writer and a fixed summation order.
 //
-// Small grids (fewer workgroups than the chip holds) split the stream of query blocks of a key block
-// over up to eight workgroups; each writes its fp32 partial dK and dV to the workspace and
-// kv_sum_kernel adds the partials in split order.
+// Small grids (fewer workgroups than the chip holds) split a key block's stream of units over up to
+// sixteen workgroups (shares of whole units, at least eight each); each writes its fp32 partial dK and
+// dV to the workspace and kv_sum_kernel adds the partials in split order.
 #include <type_traits>
 
 #include "sa2_mfma_common.h"
@@ -28,7 +28,8 @@ namespace {
 constexpr int VW = 8;                  // wavefronts per workgroup
 constexpr int VT = VW * 64;            // threads per workgroup
 constexpr int VPAIR = 4;
-constexpr int KV_MAX_SPLIT = 8;        // workgroups a key block's query blocks are split over, at most
+constexpr int KV_MAX_SPLIT = 16;       // workgroups a key block's stream of units is split over, at most
+constexpr int KV_MIN_SHARE = 8;        // units a share holds at least
 constexpr int KV_GRID_TARGET = 512;    // a split stops once the grid holds this many workgroups
 
 // KB: 32-row blocks of K/V rows per wavefront pair
@@ -61,14 +62,15 @@ struct KvCfg {
 };
 
 // BIAS = false: k2_bias and v2_bias are both zero (the reference's default), the adds drop out.
-// nsplit > 1: the workgroup takes the sp-th share of the key block's query blocks and writes fp32
+// SPLIT (nsplit > 1): the workgroup takes the sp-th share of the key block's units and writes fp32
 // partial sums to `part` ([2][nsplit][B*H][N][D]: dK before its scale, then dV).
 // SEG = true: a K' window too wide for LDS is walked in segments of ws_arg + 1 deltas; LDS holds the K'/V'
 // rows of one segment of a query block and they are reloaded at every segment.  (A kernel of its own, so that
 // the common case carries none of it.)
-template <class E, int D, bool BIAS, int KB, bool SEG>
+template <class E, int D, bool BIAS, int KB, bool SEG, bool SPLIT>
 __global__ __launch_bounds__(VT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __restrict__ part, int ws_arg) {
+void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __restrict__ part, int ws_arg) {
+    const int nsplit = nsplit_arg;           // (1 unless SPLIT; kept a run-time value: the compiler's code for the sweep is better that way)
     typedef typename E::scalar EL;
     typedef typename E::x8 X8;
     using C = KvCfg<D, KB>;
@@ -125,18 +127,35 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
     const float qscale = p.scale * LOG2E;
     const int j_last = (j0 + VJ - 1 < N ? j0 + VJ - 1 : N - 1);
     const int i_max = (int)((int64_t)j_last + w1 < N - 1 ? j_last + w1 : N - 1);
-    // the query blocks that see the key block, and this workgroup's share of them
-    int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
-    if (nsplit > 1) {
-        const int chunk = (ib_hi - ib_lo + nsplit) / nsplit;
-        ib_lo += sp * chunk;
-        ib_hi = ib_hi < ib_lo + chunk - 1 ? ib_hi : ib_lo + chunk - 1;
-    }
-    const bool has_work = ib_lo <= ib_hi;
     auto units_of = [&](int ib) {
         const int il = (ib * BQ + BQ - 1 < N ? ib * BQ + BQ - 1 : N - 1);
         return (w2 < il ? w2 : il) + 1;
     };
+    // The units (query block, delta) that see the key block, in stream order, and this workgroup's share of
+    // them: from delta d_first of block ib_lo to delta d_last of block ib_hi.  The shares cut the stream
+    // counted with w2 + 1 slots per block (a block near the start of the sequence has fewer units: the slots
+    // beyond are skipped).
+    int ib_lo = j0 / BQ, ib_hi = i_max / BQ, d_first = 0, d_last = w2;
+    bool has_work = ib_lo <= ib_hi;
+    if constexpr (SPLIT) {
+        const int per = w2 + 1, ib0 = ib_lo;
+        const int slots = (ib_hi - ib_lo + 1) * per;
+        const int chunk = (slots + nsplit - 1) / nsplit;
+        const int v_lo = sp * chunk, v_hi = (v_lo + chunk < slots ? v_lo + chunk : slots) - 1;
+        has_work = v_lo <= v_hi;
+        if (has_work) {
+            ib_lo = ib0 + v_lo / per;
+            d_first = v_lo - (ib_lo - ib0) * per;
+            ib_hi = ib0 + v_hi / per;
+            d_last = v_hi - (ib_hi - ib0) * per;
+            if (d_first >= units_of(ib_lo)) {        // the share starts in the slots a short block does not have
+                ++ib_lo;
+                d_first = 0;
+            }
+            has_work = ib_lo < ib_hi || (ib_lo == ib_hi && d_first <= d_last);
+        }
+    }
+    const int dbase0 = SEG ? d_first : 0;            // first delta of the K'/V' rows loaded first
 
     // ---- raw rows of a query block: q, dO, the K'/V' rows its deltas reach, -LSE, -D ----
     auto load_raw = [&](int ib, int dbase) {
@@ -224,17 +243,17 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
 
     // ---- prologue: first block's raw rows, first unit --------------------------------
     if (has_work) {
-        load_raw(ib_lo, 0);
+        load_raw(ib_lo, dbase0);
         __syncthreads();
         fetch_qd();
-        form(0, 0);
+        form(d_first - dbase0, 0);
         __syncthreads();
     }
 
     // The sweep, instantiated once per role so that each keeps only its own registers live.
     auto sweep = [&](auto role_tag) {
         constexpr int ROLE = decltype(role_tag)::value;
-        int ib = ib_lo, delta = 0, slot = 0, step = 0, dbase = 0;
+        int ib = ib_lo, delta = d_first, slot = 0, step = 0, dbase = dbase0;
         int nu = units_of(ib_lo);
         int cur_ib = -1;
         floatx16 negr;                               // -LSE*log2e (P) or -D (dS) of the block's rows, per accumulator element
@@ -393,7 +412,7 @@ void mfma_bwd_kv_kernel(Problem p, int njb, int total, int nsplit, float* __rest
                 nib = ib + 1;
                 ndelta = 0;
             }
-            const bool more = nib <= ib_hi;
+            const bool more = SPLIT ? (nib < ib_hi || (nib == ib_hi && ndelta <= d_last)) : nib <= ib_hi;
             const int nslot = slot + 1 == C::NUNIT ? 0 : slot + 1;
             if (more) {
                 if (nib != ib || (SEG && ndelta - dbase > ws)) {
@@ -478,11 +497,11 @@ __global__ __launch_bounds__(256) void kv_sum_kernel(Problem p, int nsplit, cons
 }
 
 // Geometry of a launch: 32-row K blocks per wavefront pair, and the number of shares a key block's
-// query blocks are split into.  Both depend on the problem's sizes only.
+// stream of units is split into.  Both depend on the problem's sizes only.
 struct KvPlan {
     int kb, nsplit;
 };
-KvPlan kv_plan(int B, int N, int H, int D, int w1) {
+KvPlan kv_plan(int B, int N, int H, int D, int w1, int w2) {
     KvPlan pl{1, 1};
     const int64_t bh = (int64_t)B * H;
     // two K blocks per pair at head_dim 64 when that still leaves a grid worth splitting no further than in two
@@ -492,7 +511,8 @@ KvPlan kv_plan(int B, int N, int H, int D, int w1) {
     const int blocks = (vj + (w1 < N ? w1 : N) + BQ - 1) / BQ + 1;          // query blocks a key block streams, at most
     // (the partial sums of a split launch stay under 32 MiB)
     auto part_bytes = [&](int ns) { return (int64_t)2 * ns * bh * N * D * 4; };
-    while (pl.nsplit < KV_MAX_SPLIT && base * pl.nsplit * 2 <= KV_GRID_TARGET && pl.nsplit * 2 <= blocks &&
+    const int64_t units = (int64_t)blocks * ((w2 < N - 1 ? w2 : N - 1) + 1);     // of a key block's stream, at most
+    while (pl.nsplit < KV_MAX_SPLIT && base * pl.nsplit * 2 <= KV_GRID_TARGET && (int64_t)pl.nsplit * 2 * KV_MIN_SHARE <= units &&
            part_bytes(pl.nsplit * 2) <= ((int64_t)32 << 20))
         pl.nsplit *= 2;
     return pl;
@@ -511,18 +531,26 @@ int launch_kv_geometry(const Problem& p, int nsplit, hipStream_t st) {
     float* part = nullptr;
     if (nsplit > 1) {
         const size_t off = kp_side_scratch_bytes(p.B, p.N, p.H, D, p.w2);
-        if (p.scratch_bytes < off + kv_split_scratch_bytes(p.B, p.N, p.H, D, p.w1)) return SA2_ERR_WORKSPACE_TOO_SMALL;
+        if (p.scratch_bytes < off + kv_split_scratch_bytes(p.B, p.N, p.H, D, p.w1, p.w2)) return SA2_ERR_WORKSPACE_TOO_SMALL;
         part = (float*)((char*)p.scratch + off);
     }
     const bool seg = ws < p.w2;
     // (the segmented kernel exists with the bias adds only)
-    const void* fn = seg    ? (const void*)mfma_bwd_kv_kernel<E, D, true, KB, true>
-                     : bias ? (const void*)mfma_bwd_kv_kernel<E, D, true, KB, false>
-                            : (const void*)mfma_bwd_kv_kernel<E, D, false, KB, false>;
-    if (!allow_full_lds(fn)) return SA2_ERR_LAUNCH_FAILED;
-    if (seg) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true, KB, true>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
-    else if (bias) hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, true, KB, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
-    else hipLaunchKernelGGL((mfma_bwd_kv_kernel<E, D, false, KB, false>), dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
+    auto go = [&](auto kernel) {
+        if (!allow_full_lds((const void*)kernel)) return false;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(VT), lds, st, p, njb, (int)total, nsplit, part, ws);
+        return true;
+    };
+    bool ok;
+    if (nsplit > 1)
+        ok = seg    ? go(mfma_bwd_kv_kernel<E, D, true, KB, true, true>)
+             : bias ? go(mfma_bwd_kv_kernel<E, D, true, KB, false, true>)
+                    : go(mfma_bwd_kv_kernel<E, D, false, KB, false, true>);
+    else
+        ok = seg    ? go(mfma_bwd_kv_kernel<E, D, true, KB, true, false>)
+             : bias ? go(mfma_bwd_kv_kernel<E, D, true, KB, false, false>)
+                    : go(mfma_bwd_kv_kernel<E, D, false, KB, false, false>);
+    if (!ok) return SA2_ERR_LAUNCH_FAILED;
     if (hipGetLastError() != hipSuccess) return SA2_ERR_LAUNCH_FAILED;
     if (nsplit > 1) {
         const int64_t chunks = (int64_t)p.B * p.H * p.N * (D / 4);
@@ -534,7 +562,7 @@ int launch_kv_geometry(const Problem& p, int nsplit, hipStream_t st) {
 
 template <class E, int D>
 int launch_kv(const Problem& p, hipStream_t st) {
-    const KvPlan pl = kv_plan(p.B, p.N, p.H, D, p.w1);
+    const KvPlan pl = kv_plan(p.B, p.N, p.H, D, p.w1, p.w2);
     if constexpr (D == 64) {
         if (pl.kb == 2) return launch_kv_geometry<E, D, 2>(p, pl.nsplit, st);
     }
@@ -543,8 +571,8 @@ int launch_kv(const Problem& p, hipStream_t st) {
 
 }  // namespace
 
-size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1) {
-    const KvPlan pl = kv_plan(B, N, H, D, w1);
+size_t kv_split_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
+    const KvPlan pl = kv_plan(B, N, H, D, w1, w2);
     return pl.nsplit > 1 ? (size_t)2 * pl.nsplit * B * H * (size_t)N * D * sizeof(float) : 0;
 }
 
