@@ -551,8 +551,8 @@ __global__ __launch_bounds__(256) void f32_dq_sum_kernel(Problem p, int nkb, con
 }
 
 // =================================================== backward, K side: dK, dV =====
-// nsplit > 1 (grids smaller than the chip): the workgroup takes the sp-th share of the key block's query
-// blocks and writes fp32 partial sums to `part` ([dK | dV][nsplit][B*H][N][D]) for f32_kv_sum_kernel.
+// nsplit > 1 (grids smaller than the chip): the workgroup takes the sp-th share of the key block's stream
+// of units and writes fp32 partial sums to `part` ([dK | dV][nsplit][B*H][N][D]) for f32_kv_sum_kernel.
 template <int D, bool SPLIT>
 __global__ __launch_bounds__(XT) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 2 : 1, D <= 64 ? 2 : 1)))
 void f32_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __restrict__ part) {
@@ -595,20 +595,39 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __r
 
     const int j_last = j0 + XJ - 1 < N ? j0 + XJ - 1 : N - 1;
     const int i_max = (int)((int64_t)j_last + w1 < N - 1 ? j_last + w1 : N - 1);
-    // the query blocks that see the key block, and this workgroup's share of them
-    int ib_lo = j0 / BQ, ib_hi = i_max / BQ;
-    if constexpr (SPLIT) {
-        const int chunk = (ib_hi - ib_lo + nsplit) / nsplit;
-        ib_lo += sp * chunk;
-        ib_hi = ib_hi < ib_lo + chunk - 1 ? ib_hi : ib_lo + chunk - 1;
-    }
-    // (a share of a split launch may be empty: it walks one block without touching it and writes zeros)
-    const bool empty_share = ib_lo > ib_hi;
-    if (empty_share) ib_lo = ib_hi = j0 / BQ;
     auto units_of = [&](int ib) {
         const int il = ib * BQ + BQ - 1 < N ? ib * BQ + BQ - 1 : N - 1;
         return (w2 < il ? w2 : il) + 1;
     };
+    // The units (query block, delta) that see the key block, in stream order, and this workgroup's share of
+    // them: from delta d_first of block ib_lo to delta d_last of block ib_hi.  The shares cut the stream
+    // counted with w2 + 1 slots per block (a block near the start of the sequence has fewer units: the slots
+    // beyond are skipped).
+    int ib_lo = j0 / BQ, ib_hi = i_max / BQ, d_first = 0, d_last = w2;
+    bool empty_share = ib_lo > ib_hi;
+    if constexpr (SPLIT) {
+        const int per = w2 + 1, ib0 = ib_lo;
+        const int slots = (ib_hi - ib_lo + 1) * per;
+        const int chunk = (slots + nsplit - 1) / nsplit;
+        const int v_lo = sp * chunk, v_hi = (v_lo + chunk < slots ? v_lo + chunk : slots) - 1;
+        empty_share = v_lo > v_hi;
+        if (!empty_share) {
+            ib_lo = ib0 + v_lo / per;
+            d_first = v_lo - (ib_lo - ib0) * per;
+            ib_hi = ib0 + v_hi / per;
+            d_last = v_hi - (ib_hi - ib0) * per;
+            if (d_first >= units_of(ib_lo)) {        // the share starts in the slots a short block does not have
+                ++ib_lo;
+                d_first = 0;
+            }
+            empty_share = !(ib_lo < ib_hi || (ib_lo == ib_hi && d_first <= d_last));
+        }
+    }
+    // (a share of a split launch may be empty: it walks one unit without touching it and writes zeros)
+    if (empty_share) {
+        ib_lo = ib_hi = j0 / BQ;
+        d_first = d_last = 0;
+    }
 
     // ---- forming a unit: Q~ and dO~ tiles (32 rows), LSE and D of its queries ----
     float4 fq[C::KR], fk[C::KR], fd[C::KR], fv[C::KR];
@@ -652,7 +671,7 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __r
         }
     };
 
-    int ib = ib_lo, delta = 0, nu = units_of(ib_lo), buf = 0;
+    int ib = ib_lo, delta = d_first, nu = units_of(ib_lo), buf = 0;
     fetch_unit(ib, delta);
     store_unit(0);
     __syncthreads();
@@ -662,7 +681,7 @@ void f32_bwd_kv_kernel(Problem p, int njb, int total, int nsplit_arg, float* __r
             nib = ib + 1;
             ndelta = 0;
         }
-        const bool more = nib <= ib_hi;
+        const bool more = SPLIT ? (nib < ib_hi || (nib == ib_hi && ndelta <= d_last)) : nib <= ib_hi;
         if (more) fetch_unit(nib, ndelta);
 
         const int i0 = ib * BQ;
@@ -768,11 +787,13 @@ __global__ __launch_bounds__(256) void f32_kv_sum_kernel(Problem p, int nsplit, 
 }
 
 // Shares a key block's query blocks are split into when the K-side grid is smaller than the chip
-int f32_kv_nsplit(int B, int N, int H, int D, int w1) {
+int f32_kv_nsplit(int B, int N, int H, int D, int w1, int w2) {
     const int64_t bh = (int64_t)B * H, base = bh * ((N + XJ - 1) / XJ);
     const int blocks = (XJ + (w1 < N ? w1 : N) + BQ - 1) / BQ + 1;
-    int ns = 1;
-    while (ns < 8 && base * ns * 2 <= 512 && ns * 2 <= blocks && (int64_t)2 * ns * 2 * bh * N * D * 4 <= ((int64_t)32 << 20)) ns *= 2;
+    const int64_t units = (int64_t)blocks * ((w2 < N - 1 ? w2 : N - 1) + 1);     // of a key block's stream, at most
+    int ns = 1;                                                                  // shares of at least 8 units
+    while (ns < 16 && base * ns * 2 <= 512 && (int64_t)ns * 2 * 8 <= units && (int64_t)2 * ns * 2 * bh * N * D * 4 <= ((int64_t)32 << 20))
+        ns *= 2;
     return ns;
 }
 size_t f32_dq_part_bytes(int B, int N, int H, int D, int w2) {
@@ -818,7 +839,7 @@ int launch_f32_bwd(const Problem& p, hipStream_t st) {
     }
     if (p.dk1.p || p.dv1.p) {
         const int njb = (p.N + XJ - 1) / XJ;
-        const int nsplit = f32_kv_nsplit(p.B, p.N, p.H, D, p.w1);
+        const int nsplit = f32_kv_nsplit(p.B, p.N, p.H, D, p.w1, p.w2);
         const int64_t total = (int64_t)njb * p.B * p.H * nsplit;
         if (total > 0x7fffffffLL) return SA2_ERR_TOO_LARGE;
         float* kv_part = nullptr;
@@ -870,7 +891,7 @@ bool f32_mfma_layout_ok(const Problem& p, bool backward) {
 }
 
 size_t f32_mfma_bwd_scratch_bytes(int B, int N, int H, int D, int w1, int w2) {
-    const int ns = f32_kv_nsplit(B, N, H, D, w1);
+    const int ns = f32_kv_nsplit(B, N, H, D, w1, w2);
     return f32_dq_part_bytes(B, N, H, D, w2) + (ns > 1 ? (size_t)2 * ns * B * H * (size_t)N * D * sizeof(float) : 0);
 }
 
