@@ -121,6 +121,13 @@ def test_config4_headline_shape_gradients():
                 more_rows=((0, 608), (8192 - 640, 8192)), label="c4 bf16 B1 H16 N8192 D128 w512/32")
 
 
+def test_segmented_k2_window_on_a_full_grid():
+    """bf16 B2 H16 N2048 D128 w 48/130: a grid that fills the chip (the K-side kernel unsplit, walking the K' rows in
+    segments of 65 deltas; the K'-side kernel with two workgroups per K' block, 112 + 19 deltas).  Oracle on the first
+    rows and the last ones, the fp32 kernels over whole tensors."""
+    check_large(2, 2048, 16, 128, 48, 130, seed=11, rows=(0, 320), more_rows=((2048 - 256, 2048),))
+
+
 def test_config5_long_sequence_gradients():
     """Benchmark configuration 5: bf16, B1 H8 N32768 D128, w 1024/64, q/k/k' ~ N(0, 0.5^2), seed 4.  Checked
     on the first query rows, rows around i = w1 and the end of the sequence, LSE included (the
