@@ -62,11 +62,11 @@ def _rows(t):
 
 def _pad_head_dim(D, dtype, flags):
     """head_dim the kernels are run with.  The MFMA kernels start at head_dim 32 (one 32-column
-    value tile); 16-bit tensors with head_dim 16 are zero-padded to 32 on the way in (zero columns
+    value tile); tensors with head_dim 16 are zero-padded to 32 on the way in (zero columns
     add nothing to a logit and give zero output and gradient columns, which are dropped again), so
-    that they take the MFMA kernels instead of the fp32 FMA kernels.  The softmax scale is always
-    the caller's (1/sqrt(16) by default), not that of the padded width."""
-    return 32 if (D == 16 and dtype in (torch.bfloat16, torch.float16) and flags == _lib.FLAG_AUTO) else D
+    that they take the MFMA kernels of their element type instead of the fp32 FMA kernels.  The
+    softmax scale is always the caller's (1/sqrt(16) by default), not that of the padded width."""
+    return 32 if (D == 16 and dtype in (torch.bfloat16, torch.float16, torch.float32) and flags == _lib.FLAG_AUTO) else D
 
 
 def _padded(t, width):
