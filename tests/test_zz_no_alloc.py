@@ -59,6 +59,8 @@ def _both_backwards(shape, w, dtype, seed, flags, inclusive=1, needs=(True,) * 5
     (torch.bfloat16, _lib.FLAG_FORCE_MFMA, ((1, 640, 4, 128), (96, 16)), ((1, 200, 2, 128), (40, 8))),
     (torch.bfloat16, _lib.FLAG_FORCE_MFMA, ((2, 512, 2, 64), (64, 32)), ((1, 96, 2, 64), (32, 5))),
     (torch.float32, _lib.FLAG_AUTO, ((1, 192, 2, 64), (32, 16)), ((1, 70, 1, 64), (16, 4))),
+    # a K' window that both backward kernels walk in segments (partial dK', dV' in the workspace too), then a plain one
+    (torch.bfloat16, _lib.FLAG_FORCE_MFMA, ((1, 260, 2, 128), (24, 180)), ((1, 130, 1, 128), (16, 12))),
 ])
 @pytest.mark.parametrize("inclusive", [1, 0])
 def test_static_workspace_backward_matches_caller_workspace(dtype, flags, first, second, inclusive):
